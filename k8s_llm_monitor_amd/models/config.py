@@ -158,7 +158,8 @@ class MoESpec:
 
 @dataclass(frozen=True)
 class DenseSpec:
-    """Plain feed-forward of width ``ff`` (up-projection, activation, down-projection)."""
+    """Dense feed-forward of width ``ff`` (up-projection, activation, down-projection; gated in
+    designs whose ``ffn`` trait says so)."""
 
     ff: int
 
@@ -192,6 +193,8 @@ class HybridConfig:
     max_position: int = 2048
     norm_eps: float = 1e-5
     logit_scale: float = 1.0
+    residual_mult: float = 1.0  # every sublayer's result is scaled by this before it joins the stream
+    logit_softcap: float = 0.0  # > 0: logits <- cap * tanh(logits / cap)
     loop: Optional[tuple] = None  # (start, stop, times): layers start .. stop-1 run `times` times
     bos_id: int = 1
     eos_ids: tuple = (2,)
@@ -235,15 +238,29 @@ class HybridConfig:
 #   depth_average  the input of layer i + 1 is a learned combination (``l<i>.dwa``) of the embedding
 #                  output and the results of layers 0 .. i
 #   ffn            the feed-forward family: "swiglu_topk" (gated experts, biased router, softmax over
-#                  the chosen logits, sigmoid-gated shared expert) or "plain_softmax" (ungated
+#                  the chosen logits, sigmoid-gated shared expert), "plain_softmax" (ungated
 #                  experts with erf-GELU, softmax over all logits and the chosen probabilities
-#                  used as they are, ungated shared expert, dense layers with xIELU)
+#                  used as they are, ungated shared expert, dense layers with xIELU) or "gated_gelu"
+#                  (dense layers down(gelu_tanh(gate h) * up h))
 #   max_position   positions a model accepts when its config.json does not say
+# and, where present (absent = the first value):
+#   scalar_norm    False / True: a block or final norm's weight is one number for all coordinates
+#   gated_residual False / True: every sublayer's result is multiplied elementwise by
+#                  sigmoid(W h + b) of the sublayer's input (``l<i>.rg1`` / ``.rg2`` and ``.b``)
+#   mixers         config ``type`` -> entry of models/hybrid.py MIXERS where the design's mixer of that
+#                  name is not the entry of the same name
+#   latent         what the design fixes for latent attention: ``rotary`` "half" (entry i turns with
+#                  i + n/2) / "pairs" (2i with 2i + 1), ``sink`` True (a learned logit per head in the
+#                  softmax denominator) / False
 DESIGN_TRAITS = {
     "dunesun": dict(block="parallel", one_plus_norm=True, learned_pos=True, token_shift=False,
                     depth_average=False, ffn="swiglu_topk", max_position=2048),
     "kisutar": dict(block="sequential", one_plus_norm=False, learned_pos=False, token_shift=True,
                     depth_average=True, ffn="plain_softmax", max_position=1 << 17),
+    "bitonex": dict(block="sequential", one_plus_norm=False, learned_pos=False, token_shift=False,
+                    depth_average=False, ffn="gated_gelu", max_position=1 << 17, scalar_norm=True,
+                    gated_residual=True, mixers={"attention": "rotary_attention"},
+                    latent=dict(rotary="pairs", sink=False)),
 }
 
 
@@ -252,14 +269,15 @@ def _flat(d: dict, prefix: str = "") -> list:
     for k, v in d.items():
         if isinstance(v, dict):
             out += _flat(v, prefix + k + ".")
-        else:
-            out.append((prefix + k, v))
+        else:  # a list (one number per head) becomes a tuple: the spec stays hashable
+            out.append((prefix + k, tuple(v) if isinstance(v, list) else v))
     return out
 
 
 def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig:
     """A :class:`HybridConfig` from a layer-list ``config.json``: ``architecture``, ``vocab``,
-    ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``loop`` {start, stop, times} and
+    ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``logit_softcap``, ``residual_mult``,
+    ``loop`` {start, stop, times} and
     ``layers`` [{type, mixer {...}, mlp {kind: moe, expert.ff, router.experts, router.top, shared.ff}
     | {kind: dense, ff} | null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
     arch = str(c["architecture"]).lower()
@@ -288,7 +306,9 @@ def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig
     return HybridConfig(name=name or arch, arch=arch, vocab_size=V, d_model=int(c["width"]),
                         layers=tuple(layers),
                         max_position=int(c.get("max_positions", DESIGN_TRAITS[arch]["max_position"])),
-                        norm_eps=float(c["norm"]["eps"]), logit_scale=float(c.get("logit_scale", 1.0)), loop=loop,
+                        norm_eps=float(c["norm"]["eps"]), logit_scale=float(c.get("logit_scale", 1.0)),
+                        residual_mult=float(c.get("residual_mult", 1.0)),
+                        logit_softcap=float(c.get("logit_softcap") or 0.0), loop=loop,
                         bos_id=int(c.get("bos_id", min(1, V - 1))), eos_ids=tuple(c.get("eos_ids", (min(2, V - 1),))))
 
 
@@ -301,7 +321,7 @@ def hybrid_config_to_dict(c: HybridConfig) -> dict:
             parts = k.split(".")
             for p in parts[:-1]:
                 cur = cur.setdefault(p, {})
-            cur[parts[-1]] = v
+            cur[parts[-1]] = list(v) if isinstance(v, tuple) else v
         return out
 
     layers = []
@@ -316,6 +336,10 @@ def hybrid_config_to_dict(c: HybridConfig) -> dict:
     d = {"architecture": c.arch.capitalize(), "vocab": c.vocab_size, "width": c.d_model, "layers": layers,
          "max_positions": c.max_position, "norm": {"eps": c.norm_eps}, "logit_scale": c.logit_scale,
          "bos_id": c.bos_id, "eos_ids": list(c.eos_ids)}
+    if c.residual_mult != 1.0:
+        d["residual_mult"] = c.residual_mult
+    if c.logit_softcap:
+        d["logit_softcap"] = c.logit_softcap
     if c.loop:
         d["loop"] = {"start": c.loop[0], "stop": c.loop[1], "times": c.loop[2]}
     return d
@@ -337,6 +361,15 @@ def _latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, window, scale, base=1000
     if kv_from is not None:
         m["kv_from"] = kv_from
     return LayerSpec("latent_attention", tuple(sorted(m.items())))
+
+
+def _rot_attn(heads, kv_heads, dim, vdim, rot_dims, base, scale):
+    return LayerSpec("attention", tuple(sorted({"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                                                "rot.dims": rot_dims, "rot.base": base, "scale": scale}.items())))
+
+
+def _lightning(heads, dim, vdim, decay):
+    return LayerSpec("lightning", tuple(sorted({"heads": heads, "dim": dim, "vdim": vdim, "decay": tuple(decay)}.items())))
 
 
 def _with_mlp(s: LayerSpec, m) -> LayerSpec:
@@ -362,3 +395,13 @@ KISUTAR_TINY = _reg(HybridConfig(
             _with_mlp(_latent(4, 16, 16, 32, 32, 40, 28, 0.2, kv_from=1), None),
             _with_mlp(_latent(2, 24, 16, 24, 24, 40, 9, 0.17, kv_from=1), MoESpec(4, 3, 32, 0))),
     max_position=4096, norm_eps=1e-6, bos_id=1, eos_ids=(2,)))
+
+# Small Bitonex-design model for CPU tests and GPU smoke runs (random weights): rotary grouped-query
+# attention, fixed-decay linear attention and latent attention, the last layer reading layer 1's latent.
+BITONEX_TINY = _reg(HybridConfig(
+    name="bitonex-tiny", arch="bitonex", vocab_size=320, d_model=80,
+    layers=(_with_mlp(_rot_attn(4, 2, 24, 16, 12, 10000.0, 0.21), DenseSpec(112)),
+            _with_mlp(_latent(3, 16, 8, 24, 40, 24, 0, 0.2, base=5000.0), DenseSpec(96)),
+            _with_mlp(_lightning(2, 24, 40, (0.9, 0.97)), None),
+            _with_mlp(_latent(2, 24, 8, 16, 32, 24, 0, 0.18, base=5000.0, kv_from=1), DenseSpec(64))),
+    max_position=4096, norm_eps=1e-6, residual_mult=0.4, logit_softcap=20.0, bos_id=1, eos_ids=(2,)))

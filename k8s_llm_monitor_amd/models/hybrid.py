@@ -1,10 +1,20 @@
 """Layer-list decoders: every layer names its token mixer (windowed attention with a softmax
-sink, the Mamba-2 recurrence, or latent attention) and an optional feed-forward; a span of layers
-may run several times with shared weights.  ``Dunesun`` and ``Kisutar`` are the designs served;
-mixers are registered by name (``MIXERS``) and feed-forward families by the design's ``ffn`` trait
-(``FFNS``), with their sizes and constants read from the layer's spec, so another layer-list
-design can reuse them in another order.  What a design fixes (block form, norm form, positions,
-token shift, depth average) is models/config.DESIGN_TRAITS.
+sink, the Mamba-2 recurrence, latent attention, rotary grouped-query attention or fixed-decay
+linear attention) and an optional feed-forward; a span of layers may run several times with shared
+weights.  ``Dunesun``, ``Kisutar`` and ``Bitonex`` are the designs served; mixers are registered by
+name (``MIXERS``) and feed-forward families by the design's ``ffn`` trait (``_ffn_for``), with their
+sizes and constants read from the layer's spec, so another layer-list design can reuse them in
+another order.  What a design fixes (block form, norm form, positions, token shift, depth average,
+gated residual, rotation layout) is models/config.DESIGN_TRAITS.
+
+Bitonex, per layer (sequential block): ``x += m * mixer(h) * sigmoid(R1 h + b1)`` with
+``h = norm1(x)``, then the same with the feed-forward, ``norm2``, ``R2`` and ``b2`` (gated
+residual; ``m`` = ``residual_mult``; a norm's weight is one number).  The gate's projection rides
+as extra rows of the sublayer's own input projection (one GEMM), and the gated sum is folded into
+the next norm's launch (ops.hybrid.gated_add_norm).  Its mixers: grouped-query attention with rotary
+positions on part of each head, a temperature per head and a sigmoid output gate; linear attention
+with a fixed decay per head as an fp32 recurrence over per-sequence state slots; latent attention
+without window or sink.  Logits are soft-capped.
 
 Kisutar, per layer (sequential block): ``x += mixer(shift(norm1(x)))``, then ``x += ff(norm2(x))``.
 ``shift`` moves every row towards the previous token's (per-channel learned fractions; the last
@@ -84,7 +94,8 @@ class WindowAttention:
 
     kind = "attention"
 
-    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str):
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None):
         m = spec.m
         self.H, self.G, self.dk, self.dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         if self.H % self.G:
@@ -135,8 +146,10 @@ class Mamba2Mixer:
     the out-projection."""
 
     kind = "mamba2"
+    stateful = True
 
-    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str):
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None):
         m = spec.m
         self.nh, self.P, self.N = int(m["heads"]), int(m["vdim"]), int(m["state"])
         self.G, self.taps, self.ng = int(m.get("groups", 1)), int(m["conv"]), int(m.get("norm_groups", 1))
@@ -174,13 +187,21 @@ class Mamba2Mixer:
 class LatentAttention:
     """Attention over a compressed key/value stream (one normed latent of ``kv_rank`` and one
     rotated key part of ``rot_dim`` per token, shared by all heads), rotary positions on the
-    ``rot_dim`` part of queries and keys, a sliding window and a learned per-head sink.
-    ``kv_from``: j - no key/value projection of its own; reads layer j's pages."""
+    ``rot_dim`` part of queries and keys, a sliding window (``mask.size``; 0 / absent: none) and -
+    where the design has one - a learned per-head sink.  The design's ``latent`` trait fixes the
+    rotation layout (``rotary`` "half" / "pairs") and ``sink``.
+    ``kv_from``: j - no key/value projection of its own; reads layer j's pages.
+    ``tail``: extra rows [n, d] for the down-projection; forward leaves their outputs in ``tail_out``
+    (a [T, n] view) - the block's residual gate rides in the mixer's first GEMM."""
 
     kind = "latent_attention"
 
-    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str):
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None):
         m = spec.m
+        lt = (traits or {}).get("latent", {})
+        self.pairs = lt.get("rotary", "half") == "pairs"
+        self.sink = bool(lt.get("sink", True))
         self.H, self.dn, self.dr, self.dv = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"])
         self.Q, self.R = int(m["q_rank"]), int(m["kv_rank"])
         self.scale = float(m.get("scale", 1.0 / math.sqrt(self.dn + self.dr)))
@@ -199,12 +220,17 @@ class LatentAttention:
         if self.kv_from is None:
             wd.append(p.get(prefix + "dkv", (R + dr, d), 1.0 / math.sqrt(d)))
             self.kn = p.get(prefix + "dkv.norm", (R,), 0.1, 1.0, small=True)
-        self.w_down = torch.cat(wd).contiguous()  # [q_rank (+ kv_rank + rot_dim), d]: one launch
+        self.n_down = sum(w.shape[0] for w in wd)
+        self.n_tail = 0 if tail is None else tail.shape[0]
+        if tail is not None:
+            wd.append(tail)
+        self.tail_out = None
+        self.w_down = torch.cat(wd).contiguous()  # [q_rank (+ kv_rank + rot_dim) (+ tail), d]: one launch
         self.qn = p.get(prefix + "dq.norm", (Q,), 0.1, 1.0, small=True)
         self.w_uq = p.get(prefix + "uq", (H * (dn + dr), Q), 1.0 / math.sqrt(Q))
         self.w_uk = p.get(prefix + "uk", (H * dn, R), 1.0 / math.sqrt(R))  # viewed [H, dn, R]
         self.w_uv = p.get(prefix + "uv", (H * dv, R), 1.0 / math.sqrt(R))  # viewed [H, dv, R]
-        self.sinks = p.get(prefix + "sink", (H,), 1.0, small=True)
+        self.sinks = p.get(prefix + "sink", (H,), 1.0, small=True) if self.sink else None
         self.freq = hops.rotary_freq(self.base, self.rdims, p.device)
         self.wo = p.get(prefix + "o", (d, H * dv), 1.0 / math.sqrt(H * dv))
 
@@ -222,24 +248,26 @@ class LatentAttention:
         H, dn, dr, dv, Q, R = self.H, self.dn, self.dr, self.dv, self.Q, self.R
         T = h.shape[0]
         down = F.linear(h, self.w_down)
+        if self.n_tail:
+            self.tail_out = (down, self.n_down)
+            down = down[:, :self.n_down]
         kc, vc = cache["k"], cache["v"]
         own = self.kv_from is None
         hops.latent_prep(down, Q, R, dr, self.qn, self.kn, self.eps, meta.positions, self.freq,
-                         kc if own else None, vc if own else None, meta.slot_mapping if own else None)
+                         kc if own else None, vc if own else None, meta.slot_mapping if own else None, pairs=self.pairs)
         q = F.linear(down[:, :Q], self.w_uq)
         # the per-head key expansion moved to the query: q_lat[h] = q_unrotated[h] @ W_uk[h]  ([H, T, R])
         q_lat = torch.bmm(q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1), self.w_uk.view(H, dn, R))
-        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq, self.pitch)
+        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq, self.pitch, pairs=self.pairs)
         args = (H, self.scale, self.window, self.sinks)
+        kw = dict(fast=self.fast, sink=self.sink)
         if not meta.is_prefill:
-            o = hops.latent_attention(qa, kc, vc, meta.block_tables, *args, seq_lens=meta.seq_lens, fast=self.fast)
+            o = hops.latent_attention(qa, kc, vc, meta.block_tables, *args, seq_lens=meta.seq_lens, **kw)
         else:
             nd = meta.num_decode
-            o = hops.latent_attention(qa[nd:], kc, vc, meta.block_tables, *args, cu=meta.cu_seqlens, ctx=meta.ctx_start,
-                                      fast=self.fast)
+            o = hops.latent_attention(qa[nd:], kc, vc, meta.block_tables, *args, cu=meta.cu_seqlens, ctx=meta.ctx_start, **kw)
             if nd:
-                od = hops.latent_attention(qa[:nd], kc, vc, meta.dec_block_tables, *args, seq_lens=meta.dec_seq_lens,
-                                           fast=self.fast)
+                od = hops.latent_attention(qa[:nd], kc, vc, meta.dec_block_tables, *args, seq_lens=meta.dec_seq_lens, **kw)
                 o = torch.cat([od, o])
         # ... and the value expansion to the result: v[h] = o_lat[h] @ W_uv[h]^T, written head by head
         # into the rows the out-projection reads
@@ -248,7 +276,128 @@ class LatentAttention:
         return F.linear(v.view(T, H * dv), self.wo)
 
 
-MIXERS = {WindowAttention.kind: WindowAttention, Mamba2Mixer.kind: Mamba2Mixer, LatentAttention.kind: LatentAttention}
+class RotaryAttention:
+    """Grouped-query softmax attention with rotary positions on the first ``rot.dims`` entries of every
+    query / key head (entry i turns with entry i + rot.dims / 2; frequencies ``rot.base^(-2i/dims)``),
+    a learned temperature per query head (``temp``: score = q.k * scale * temp[h]) and a sigmoid
+    output gate ``heads * sigmoid(G h)`` in front of the out-projection.  Causal; ``mask.size`` keys
+    of sliding window where given (0 / absent: all).  Pages and attention kernels are windowed
+    attention's; the temperature is folded into the query in the rotation pass.
+    ``tail``: extra rows for the input projection (see LatentAttention)."""
+
+    kind = "rotary_attention"
+
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None):
+        m = spec.m
+        self.H, self.G, self.dk, self.dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+        if self.H % self.G:
+            raise ValueError(f"{prefix}: heads {self.H} not a multiple of kv_heads {self.G}")
+        self.scale = float(m.get("scale", 1.0 / math.sqrt(self.dk)))
+        self.window = int(m.get("mask.size", 0) or 0)
+        self.base, self.rdims = float(m.get("rot.base", 10000.0)), int(m.get("rot.dims", self.dk))
+        if self.rdims % 2 or not 0 <= self.rdims <= self.dk:
+            raise ValueError(f"{prefix}: rot.dims {self.rdims} must be even and at most dim {self.dk}")
+        self.pairs = (traits or {}).get("attention_rotary", "half") == "pairs"
+        self.fast = 1
+        nq, nk, nv = self.H * self.dk, self.G * self.dk, self.G * self.dv
+        s = 1.0 / math.sqrt(d)
+        ws = [p.get(prefix + "q", (nq, d), s), p.get(prefix + "k", (nk, d), s), p.get(prefix + "v", (nv, d), s),
+              p.get(prefix + "g", (self.H * self.dv, d), s)]
+        self.g_col = nq + nk + nv
+        self.n_in = self.g_col + self.H * self.dv
+        self.n_tail = 0 if tail is None else tail.shape[0]
+        if tail is not None:
+            ws.append(tail)
+        self.tail_out = None
+        self.w_in = torch.cat(ws).contiguous()  # [q | k | v | gate (| tail)]: one launch
+        self.temp = p.get(prefix + "temp", (self.H,), 0.2, 1.0, small=True)
+        self.freq = hops.rotary_freq(self.base, self.rdims, p.device)
+        self.wo = p.get(prefix + "o", (d, self.H * self.dv), 1.0 / math.sqrt(self.H * self.dv))
+
+    def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
+        return {"k": torch.zeros(num_blocks, BLOCK, self.G * self.dk, dtype=dtype, device=device),
+                "v": torch.zeros(num_blocks, self.G, self.dv, BLOCK, dtype=dtype, device=device)}
+
+    def cache_bytes(self, esize: int) -> tuple:
+        return BLOCK * self.G * (self.dk + self.dv) * esize, 0
+
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict) -> torch.Tensor:
+        H, G, dk, dv = self.H, self.G, self.dk, self.dv
+        proj = F.linear(h, self.w_in)
+        if self.n_tail:
+            self.tail_out = (proj, self.n_in)
+        kc, vc = cache["k"], cache["v"]
+        hops.rotary_cache(proj, H, G, dk, dv, meta.positions, self.freq, self.pairs, self.temp, kc, vc, meta.slot_mapping)
+        args = (H, G, dk, dv, self.scale, self.window, False)
+        if not meta.is_prefill:
+            o = hops.window_attention_decode(proj, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast))
+        else:
+            nd = meta.num_decode
+            o = hops.window_attention_prefill(proj[nd:], kc, vc, meta.cu_seqlens, meta.ctx_start, meta.block_tables,
+                                              *args, mfma=self.fast)
+            if nd:
+                od = hops.window_attention_decode(proj[:nd], kc, vc, meta.dec_block_tables, meta.dec_seq_lens, *args,
+                                                  vec=bool(self.fast))
+                o = torch.cat([od, o])
+        return F.linear(hops.sigmoid_gate(o, proj, self.g_col), self.wo)
+
+
+class LightningMixer:
+    """Linear attention with a fixed decay per head: ``q, k, v = silu(projections)``; per head
+    ``S_t = decay[h] S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` (no other scale); all heads' outputs
+    are RMS-normed together (weight ``norm``), multiplied by ``sigmoid(G h)`` and projected.  The
+    state [heads, dim, vdim] is fp32, one per sequence slot, carried from step to step; it is the
+    recurrence of ops.hybrid.ssm_scan with a constant decay, step size 1 and no skip term.
+    ``tail``: extra rows for the input projection (see LatentAttention)."""
+
+    kind = "lightning"
+    stateful = True
+
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None):
+        m = spec.m
+        self.H, self.dk, self.dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        dec = m["decay"]
+        dec = [float(dec)] * self.H if isinstance(dec, (int, float)) else [float(x) for x in dec]
+        if len(dec) != self.H:
+            raise ValueError(f"{prefix}: {len(dec)} decays for {self.H} heads")
+        self.eps = eps
+        H, dk, dv = self.H, self.dk, self.dv
+        s = 1.0 / math.sqrt(d)
+        # rows [v | k | q | gate (| tail)]: the recurrence reads x, B, C = v, k, q in that order
+        ws = [p.get(prefix + "v", (H * dv, d), s), p.get(prefix + "k", (H * dk, d), s), p.get(prefix + "q", (H * dk, d), s),
+              p.get(prefix + "g", (H * dv, d), s)]
+        self.n_act = H * dv + 2 * H * dk
+        self.n_in = self.n_act + H * dv
+        self.n_tail = 0 if tail is None else tail.shape[0]
+        if tail is not None:
+            ws.append(tail)
+        self.tail_out = None
+        self.w_in = torch.cat(ws).contiguous()
+        self.decay = torch.tensor(dec, dtype=torch.float32, device=p.device)
+        self.norm_w = p.get(prefix + "norm", (H * dv,), 0.1, 1.0, small=True)
+        self.wo = p.get(prefix + "o", (d, H * dv), 1.0 / math.sqrt(H * dv))
+
+    def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
+        return {"state": torch.zeros(num_slots, self.H, self.dk, self.dv, dtype=torch.float32, device=device)}
+
+    def cache_bytes(self, esize: int) -> tuple:
+        return 0, self.H * self.dk * self.dv * 4
+
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict) -> torch.Tensor:
+        proj = F.linear(h, self.w_in)
+        if self.n_tail:
+            self.tail_out = (proj, self.n_in)
+        vkq = hops.activation_cols(proj, 0, self.n_act, "silu")
+        o = hops.linear_attention(vkq, self.decay, cache["state"], meta.seg_cu, meta.seg_ctx, meta.seg_slot,
+                                  self.H, self.dk, self.dv)
+        g = hops.gated_group_norm(o, proj, self.n_act, self.norm_w, self.eps, 1, h.dtype, after=True)
+        return F.linear(g, self.wo)
+
+
+MIXERS = {WindowAttention.kind: WindowAttention, Mamba2Mixer.kind: Mamba2Mixer, LatentAttention.kind: LatentAttention,
+          RotaryAttention.kind: RotaryAttention, LightningMixer.kind: LightningMixer}
 
 
 class RoutedFFN:
@@ -306,6 +455,28 @@ class DenseFFN:
         return F.linear(hops.activation(F.linear(h, self.w_up), "xielu", self.a_pos, self.a_neg), self.w_down)
 
 
+class GatedDenseFFN:
+    """``down(gelu_tanh(gate h) * (up h))``: gate and up (and ``tail``: extra rows whose outputs
+    forward leaves in ``tail_out``) in one projection, the gated unit in one launch."""
+
+    def __init__(self, spec: DenseSpec, d: int, p: _Params, prefix: str, tail: Optional[torch.Tensor] = None):
+        self.ff = spec.ff
+        s = 1.0 / math.sqrt(d)
+        ws = [p.get(prefix + "gate", (self.ff, d), s), p.get(prefix + "up", (self.ff, d), s)]
+        self.n_tail = 0 if tail is None else tail.shape[0]
+        if tail is not None:
+            ws.append(tail)
+        self.tail_out = None
+        self.w_in = torch.cat(ws).contiguous()
+        self.w_down = p.get(prefix + "down", (d, self.ff), 1.0 / math.sqrt(self.ff))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        proj = F.linear(h, self.w_in)
+        if self.n_tail:
+            self.tail_out = (proj, 2 * self.ff)
+        return F.linear(hops.glu(proj, 0, self.ff, "gelu_tanh"), self.w_down)
+
+
 class PlainRoutedFFN:
     """Top-k routed ungated experts ``down_e(gelu(up_e h))`` (erf GELU): fp32 router without bias,
     softmax over all experts, the chosen experts weighted by their probabilities as they are; plus
@@ -335,10 +506,12 @@ class PlainRoutedFFN:
         return hops.moe_experts(h, ids, wts, self.w1, self.w2, shared, None, act="gelu")
 
 
-def _ffn_for(family: str, spec, d: int, p: _Params, prefix: str):
+def _ffn_for(family: str, spec, d: int, p: _Params, prefix: str, tail: Optional[torch.Tensor] = None):
     """The feed-forward of a layer in a design's family (models/config.DESIGN_TRAITS ``ffn``)."""
     if spec is None:
         return None
+    if family == "gated_gelu" and isinstance(spec, DenseSpec):
+        return GatedDenseFFN(spec, d, p, prefix, tail)
     if family == "swiglu_topk" and isinstance(spec, MoESpec):
         return RoutedFFN(spec, d, p, prefix)
     if family == "plain_softmax":
@@ -367,8 +540,11 @@ class HybridLM:
         tr = cfg.traits
         self.sequential = tr["block"] == "sequential"
         self.one_plus, self.shifted, self.depth_avg = tr["one_plus_norm"], tr["token_shift"], tr["depth_average"]
-        if (self.shifted or self.depth_avg) and not self.sequential:
-            raise ValueError(f"{cfg.name}: token shift and depth average are built for sequential blocks")
+        self.scalar_norm, self.gated = bool(tr.get("scalar_norm")), bool(tr.get("gated_residual"))
+        if (self.shifted or self.depth_avg or self.gated) and not self.sequential:
+            raise ValueError(f"{cfg.name}: token shift, depth average and gated residual are built for sequential blocks")
+        if self.gated and (self.shifted or self.depth_avg):
+            raise ValueError(f"{cfg.name}: gated residual is not combined with token shift or depth average")
         if self.depth_avg and cfg.loop:
             raise ValueError(f"{cfg.name}: depth average over looped layers is not defined")
         nm = 1.0 if not self.one_plus else 0.0  # plain norm weights sit around one
@@ -376,19 +552,36 @@ class HybridLM:
         self.pos = p.get("pos", (cfg.max_position, d), 0.1) if tr["learned_pos"] else None
         self.loop_step = p.get("loop.step", (cfg.loop[2], d), 0.1, small=True) if cfg.loop else None
         self.norms, self.norms2, self.mixers, self.ffns, self.shifts, self.dwa = [], [], [], [], [], []
+        self.rg1, self.rg2 = [], []  # gated residual: (bias [d] fp32, weight rows kept for export), per sublayer
+        names = tr.get("mixers", {})
+        nshape = () if self.scalar_norm else (d,)
+
+        def norm_w(name):  # one number per norm is kept as a [d] vector: the norm kernels read a vector
+            w = p.get(name, nshape, 0.1, nm, small=True)
+            return w.reshape(1).expand(d).contiguous() if self.scalar_norm else w
+
+        def rgate(name):
+            return p.get(name, (d, d), 1.0 / math.sqrt(d)), p.get(name + ".b", (d,), 0.5, small=True)
+
         for i, spec in enumerate(cfg.layers):
-            if spec.kind not in MIXERS:
+            kind = names.get(spec.kind, spec.kind)
+            if kind not in MIXERS:
                 raise ValueError(f"layer {i}: unknown mixer {spec.kind!r} (known: {sorted(MIXERS)})")
-            self.norms.append(p.get(f"l{i}.norm1", (d,), 0.1, nm, small=True))
-            self.mixers.append(MIXERS[spec.kind](spec, d, cfg.norm_eps, p, f"l{i}.mix."))
-            self.ffns.append(_ffn_for(tr["ffn"], spec.mlp, d, p, f"l{i}.mlp."))
-            self.norms2.append(p.get(f"l{i}.norm2", (d,), 0.1, nm, small=True)
-                               if self.sequential and spec.mlp is not None else None)
+            self.norms.append(norm_w(f"l{i}.norm1"))
+            g1 = rgate(f"l{i}.rg1") if self.gated else None
+            self.mixers.append(MIXERS[kind](spec, d, cfg.norm_eps, p, f"l{i}.mix.", traits=tr,
+                                            tail=g1[0] if g1 else None))
+            g2 = rgate(f"l{i}.rg2") if self.gated and spec.mlp is not None else None
+            self.ffns.append(_ffn_for(tr["ffn"], spec.mlp, d, p, f"l{i}.mlp.", tail=g2[0] if g2 else None)
+                             if self.gated else _ffn_for(tr["ffn"], spec.mlp, d, p, f"l{i}.mlp."))
+            self.rg1.append(self._gate_for(self.mixers[-1], g1))
+            self.rg2.append(self._gate_for(self.ffns[-1], g2))
+            self.norms2.append(norm_w(f"l{i}.norm2") if self.sequential and spec.mlp is not None else None)
             self.shifts.append(p.get(f"l{i}.shift", (d,), 0.25, 0.4, small=True) if self.shifted else None)
             # depth-average coefficients: random init leans on the newest result so the stream stays sane
             self.dwa.append(p.get(f"l{i}.dwa", (i + 2,), 0.3 / (i + 2), 1.0 / (i + 2), small=True)
                             if self.depth_avg else None)
-        self.final_norm = p.get("final.norm", (d,), 0.1, nm, small=True)
+        self.final_norm = norm_w("final.norm")
         self.head = p.get("head", (V, d), 1.0 / math.sqrt(d))
         self.runs = cfg.runs()
         # the run whose pages a run reads: its own, or the latest earlier run of the layer it names
@@ -408,11 +601,20 @@ class HybridLM:
                 raise ValueError(f"layer {li}: kv_from {src} has not run before it")
             self.kv_run.append(prev[-1])
         self.unused = sorted(set(weights.keys()) - p.used) if weights is not None else []
-        self.has_state = self.shifted or any(m.kind == "mamba2" for m in self.mixers)
+        self.has_state = self.shifted or any(getattr(m, "stateful", False) for m in self.mixers)
         # large steps of such layers run on the Mixtral path's tile GEMM (extension _k8sllm_ops)
         self.uses_tile_gemm = any(f is not None and (getattr(f, "il", False) or getattr(f, "tile", False))
                                   for f in self.ffns)
         self.layer_probe = None  # a list: forward() appends the residual stream after every run
+
+    @staticmethod
+    def _gate_for(sub, g: Optional[tuple]) -> Optional[dict]:
+        """A sublayer's residual gate: its bias, and its weight rows where the sublayer's own input
+        projection does not carry them (``tail``) - then the gate is a projection of its own."""
+        if g is None:
+            return None
+        fused = getattr(sub, "n_tail", 0) > 0
+        return {"b": g[1], "w": None if fused else g[0]}
 
     # ------------------------------------------------------------------ engine interface
     def overlap_ok(self) -> bool:
@@ -448,6 +650,7 @@ class HybridLM:
     def _tensors(self) -> list:
         ts = [self.embed, self.final_norm, self.head] + self.norms
         ts += [t for t in [self.pos, self.loop_step] + self.norms2 + self.shifts + self.dwa if t is not None]
+        ts += [t for g in self.rg1 + self.rg2 if g is not None for t in g.values() if t is not None]
         for o in self.mixers + [f for f in self.ffns if f is not None]:
             ts += [v for v in vars(o).values() if isinstance(v, torch.Tensor)]
         return ts
@@ -478,7 +681,7 @@ class HybridLM:
             x = x.index_select(0, idx)
             pending = tuple(a.index_select(0, idx) for a in pending)
         hf = hops.add_norm(x, pending, None, self.final_norm, c.norm_eps, True, self.dtype)
-        return F.linear(hf, self.head).float() * c.logit_scale
+        return self._logits(hf)
 
     def _forward_sequential(self, ids: torch.Tensor, meta: AttnMeta, caches: list) -> torch.Tensor:
         """Pre-norm blocks with two norms.  Without depth average the stream is updated in place and
@@ -495,6 +698,8 @@ class HybridLM:
             x = stack[1]
         else:
             x = hops.embed_pos(ids, meta.positions, self.embed, self.pos, meta.dec_src, meta.dec_prev)
+        if self.gated:
+            return self._forward_gated(x, meta, caches)
         pending: tuple = ()
         for r, (li, t, first) in enumerate(self.runs):
             if first and self.loop_step is not None:
@@ -519,27 +724,95 @@ class HybridLM:
             x = x.index_select(0, idx)
             pending = tuple(a.index_select(0, idx) for a in pending)
         hf = hops.add_norm(x, pending, None, self.final_norm, c.norm_eps, self.one_plus, self.dtype)
-        return F.linear(hf, self.head).float() * c.logit_scale
+        return self._logits(hf)
+
+    def _logits(self, hf: torch.Tensor) -> torch.Tensor:
+        c = self.cfg
+        z = F.linear(hf, self.head).float()
+        if c.logit_scale != 1.0:
+            z = z * c.logit_scale
+        if c.logit_softcap > 0:
+            z = hops.softcap(z.contiguous(), c.logit_softcap)
+        return z
+
+    def _gate_of(self, sub, g: dict, h: torch.Tensor) -> tuple:
+        """(projection, first column) holding a sublayer's residual-gate logits for this step."""
+        if g["w"] is None:
+            return sub.tail_out
+        return F.linear(h, g["w"]), 0
+
+    def _forward_gated(self, x: torch.Tensor, meta: AttnMeta, caches: list) -> torch.Tensor:
+        """Sequential blocks with a gated residual: every sublayer's result y joins the stream as
+        ``x += m * y * sigmoid(gate + b)``, folded into the launch of the norm that follows it."""
+        c = self.cfg
+        eps, op, mult = c.norm_eps, self.one_plus, c.residual_mult
+        pend = None  # (y, projection holding the gate logits, their first column, bias)
+        for r, (li, t, first) in enumerate(self.runs):
+            if first and self.loop_step is not None:
+                if pend is not None:
+                    raise ValueError("looped layers with a gated residual are not built")
+                x += self.loop_step[t]
+            w1 = self.norms[li]
+            h = hops.add_norm(x, (), None, w1, eps, op, self.dtype) if pend is None else \
+                hops.gated_add_norm(x, pend[0], pend[1], pend[2], pend[3], mult, w1, eps, op, self.dtype)
+            mx = self.mixers[li]
+            y = mx.forward(h, meta, caches[self.kv_run[r]])
+            pend = (y, *self._gate_of(mx, self.rg1[li], h), self.rg1[li]["b"])
+            ff = self.ffns[li]
+            if ff is not None:
+                h2 = hops.gated_add_norm(x, pend[0], pend[1], pend[2], pend[3], mult, self.norms2[li], eps, op, self.dtype)
+                y = ff.forward(h2)
+                pend = (y, *self._gate_of(ff, self.rg2[li], h2), self.rg2[li]["b"])
+            if self.layer_probe is not None:
+                d = x.shape[1]
+                g = pend[1][:, pend[2]:pend[2] + d].float() + pend[3].float()
+                self.layer_probe.append(x + mult * pend[0].float() * torch.sigmoid(g))
+        if meta.logits_idx is not None:
+            idx, d = meta.logits_idx, x.shape[1]
+            x = x.index_select(0, idx)
+            if pend is not None:
+                pend = (pend[0].index_select(0, idx), pend[1][:, pend[2]:pend[2] + d].index_select(0, idx), 0, pend[3])
+        hf = hops.add_norm(x, (), None, self.final_norm, eps, op, self.dtype) if pend is None else \
+            hops.gated_add_norm(x, pend[0], pend[1], pend[2], pend[3], mult, self.final_norm, eps, op, self.dtype)
+        return self._logits(hf)
 
 
 def state_dict(model: HybridLM) -> dict:
     """name -> tensor under the checkpoint's names (exporting a random-init model)."""
-    out = {"embed": model.embed, "final.norm": model.final_norm, "head": model.head}
+    one = (lambda w: w[0]) if model.scalar_norm else (lambda w: w)  # a one-number norm is kept as a vector
+    out = {"embed": model.embed, "final.norm": one(model.final_norm), "head": model.head}
     if model.pos is not None:
         out["pos"] = model.pos
     if model.loop_step is not None:
         out["loop.step"] = model.loop_step
     for i, (n, m, f) in enumerate(zip(model.norms, model.mixers, model.ffns)):
         p = f"l{i}."
-        out[p + "norm1"] = n
-        for key, t in (("norm2", model.norms2[i]), ("shift", model.shifts[i]), ("dwa", model.dwa[i])):
+        out[p + "norm1"] = one(n)
+        if model.norms2[i] is not None:
+            out[p + "norm2"] = one(model.norms2[i])
+        for key, t in (("shift", model.shifts[i]), ("dwa", model.dwa[i])):
             if t is not None:
                 out[p + key] = t
+        for key, g, sub in (("rg1", model.rg1[i], m), ("rg2", model.rg2[i], f)):
+            if g is not None:  # the gate's rows are the tail of the sublayer's input projection, or its own
+                w_in = getattr(sub, "w_in", getattr(sub, "w_down", None))
+                out[p + key] = g["w"] if g["w"] is not None else w_in[w_in.shape[0] - sub.n_tail:]
+                out[p + key + ".b"] = g["b"]
         if isinstance(m, LatentAttention):
             out.update({p + "mix.dq": m.w_down[:m.Q], p + "mix.dq.norm": m.qn, p + "mix.uq": m.w_uq, p + "mix.uk": m.w_uk,
-                        p + "mix.uv": m.w_uv, p + "mix.sink": m.sinks, p + "mix.o": m.wo})
+                        p + "mix.uv": m.w_uv, p + "mix.o": m.wo})
+            if m.sinks is not None:
+                out[p + "mix.sink"] = m.sinks
             if m.kv_from is None:
-                out.update({p + "mix.dkv": m.w_down[m.Q:], p + "mix.dkv.norm": m.kn})
+                out.update({p + "mix.dkv": m.w_down[m.Q:m.n_down], p + "mix.dkv.norm": m.kn})
+        elif isinstance(m, RotaryAttention):
+            nq, nk, nv = m.H * m.dk, m.G * m.dk, m.G * m.dv
+            out.update({p + "mix.q": m.w_in[:nq], p + "mix.k": m.w_in[nq:nq + nk], p + "mix.v": m.w_in[nq + nk:m.g_col],
+                        p + "mix.g": m.w_in[m.g_col:m.n_in], p + "mix.temp": m.temp, p + "mix.o": m.wo})
+        elif isinstance(m, LightningMixer):
+            nv, nk = m.H * m.dv, m.H * m.dk
+            out.update({p + "mix.v": m.w_in[:nv], p + "mix.k": m.w_in[nv:nv + nk], p + "mix.q": m.w_in[nv + nk:m.n_act],
+                        p + "mix.g": m.w_in[m.n_act:m.n_in], p + "mix.norm": m.norm_w, p + "mix.o": m.wo})
         elif isinstance(m, WindowAttention):
             nq, nk = m.H * m.dk, m.G * m.dk
             out.update({p + "mix.q": m.wqkv[:nq], p + "mix.k": m.wqkv[nq:nq + nk], p + "mix.v": m.wqkv[nq + nk:],
@@ -548,7 +821,9 @@ def state_dict(model: HybridLM) -> dict:
             out.update({p + "mix.in": m.w_in, p + "mix.conv": m.conv_w, p + "mix.conv.b": m.conv_b,
                         p + "mix.dt_bias": m.dt_bias, p + "mix.A_log": m.a_log, p + "mix.D": m.d_skip,
                         p + "mix.norm": m.norm_w, p + "mix.o": m.wo})
-        if isinstance(f, DenseFFN):
+        if isinstance(f, GatedDenseFFN):
+            out.update({p + "mlp.gate": f.w_in[:f.ff], p + "mlp.up": f.w_in[f.ff:2 * f.ff], p + "mlp.down": f.w_down})
+        elif isinstance(f, DenseFFN):
             out.update({p + "mlp.up": f.w_up, p + "mlp.down": f.w_down, p + "mlp.act": f.act})
         elif isinstance(f, PlainRoutedFFN):
             for e in range(f.E):

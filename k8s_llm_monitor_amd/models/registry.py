@@ -17,7 +17,7 @@ from .hybrid import HybridLM
 from .llama import CausalLM
 
 # config.arch -> model class
-MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM, "kisutar": HybridLM}
+MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM, "kisutar": HybridLM, "bitonex": HybridLM}
 # layer-list designs by the ``architecture`` value of their config.json (lower case)
 LAYER_LIST_ARCHS = set(DESIGN_TRAITS)
 

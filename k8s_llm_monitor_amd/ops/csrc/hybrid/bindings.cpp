@@ -12,7 +12,18 @@ int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const
                        int t2, const float* vec, const float* w, long rows, int d, float eps, int one_plus, int f32,
                        hipStream_t s);
 int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_stride, const float* w, long rows,
-                               int n, int groups, float eps, int f32, hipStream_t s);
+                               int n, int groups, float eps, int after, int f32, hipStream_t s);
+int k8sllm_hy_gated_add_norm(void* out, float* residual, const void* y, int yt, const void* gate, long g_stride,
+                             const float* bias, float mult, const float* w, long rows, int d, float eps, int one_plus,
+                             int vec, int f32, hipStream_t s);
+int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, int vec, int f32, hipStream_t s);
+int k8sllm_hy_activation_cols(void* out, const void* x, long x_stride, long rows, int n, int kind, int vec, int f32,
+                              hipStream_t s);
+int k8sllm_hy_sigmoid_gate(void* x, const void* z, long z_stride, long rows, int n, int vec, int f32, hipStream_t s);
+int k8sllm_hy_softcap(float* x, long n, float cap, hipStream_t s);
+int k8sllm_hy_rotary_cache(void* qkv, long stride, long T, int Hq, int G, int dk, int dv, const int* positions,
+                           const float* freq, int nf, int pairs, const float* q_scale, void* k_cache, void* v_cache,
+                           const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_swiglu(void* out, const void* gu, long rows, int f, int f32, hipStream_t s);
 int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float* kw, float eps, long T, int nq,
                             int nk, int nv, void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
@@ -28,8 +39,9 @@ int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int 
                         int taps, void* state, const int* cu, const int* ctx, const int* slot, int S, long T, int f32,
                         hipStream_t s);
 int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
-                       const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
-                       const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode, hipStream_t s);
+                       const float* a_log, const float* d_skip, const float* decay, float* state, const int* cu,
+                       const int* ctx, const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode,
+                       hipStream_t s);
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
                      const float* bias, int E, int K, int rows_w, int over_all, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
@@ -44,10 +56,11 @@ int k8sllm_hy_depth_mix(float* stack, long plane, int n, const void* addend, int
                         hipStream_t s);
 int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, float b, int f32, hipStream_t s);
 int k8sllm_hy_latent_prep(void* proj, long stride, long T, int Q, int R, int dr, const float* qw, const float* kw,
-                          float eps, const int* positions, const float* freq, int nf, void* k_cache, int kw_pitch,
-                          void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
+                          float eps, const int* positions, const float* freq, int nf, int pairs, void* k_cache,
+                          int kw_pitch, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_latent_queries(void* out, const void* q, long q_stride, const void* q_lat, long T, int H, int dn, int dr,
-                             int R, int w, const int* positions, const float* freq, int nf, int f32, hipStream_t s);
+                             int R, int w, const int* positions, const float* freq, int nf, int pairs, int f32,
+                             hipStream_t s);
 int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const void* k_cache, const void* v_cache,
                                const int* cu, const int* ctx, const int* seq_lens, const int* block_tables,
                                int bt_stride, int S, long T, int H, int dkp, int dv, int bs, float scale, int window,
@@ -133,7 +146,8 @@ void add_norm(Tensor out, Tensor residual, OptT a0, OptT a1, OptT a2, OptT vec, 
         "add_norm");
 }
 
-void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w, double eps, int64_t groups) {
+void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w, double eps, int64_t groups,
+                      bool after) {
   const int f = act(out, "out");
   same(proj, f, "proj");
   f32c(y, "y");
@@ -145,8 +159,80 @@ void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w
               "gated_group_norm: shapes");
   check(k8sllm_hy_gated_group_norm(out.data_ptr(), y.data_ptr<float>(),
                                    (const char*)proj.data_ptr() + z_col * proj.element_size(), proj.stride(0),
-                                   w.data_ptr<float>(), y.size(0), (int)n, (int)groups, (float)eps, f, cur()),
+                                   w.data_ptr<float>(), y.size(0), (int)n, (int)groups, (float)eps, after, f, cur()),
         "gated_group_norm");
+}
+
+// true when 8-wide accesses of a column range [col, col + n) of rows `stride` apart are aligned
+bool vec8(const Tensor& t, int64_t col, int64_t n) {
+  return n % 8 == 0 && col % 8 == 0 && t.stride(0) % 8 == 0 &&
+         reinterpret_cast<uintptr_t>(t.data_ptr()) % (8 * t.element_size()) == 0;
+}
+
+void gated_add_norm(Tensor out, Tensor residual, Tensor y, Tensor proj, int64_t g_col, Tensor bias, double mult, Tensor w,
+                    double eps, bool one_plus) {
+  const int f = act(out, "out");
+  same(proj, f, "gate");
+  f32c(residual, "residual");
+  f32c(w, "w");
+  f32c(bias, "gate bias");
+  TORCH_CHECK(residual.dim() == 2 && out.is_contiguous() && out.numel() == residual.numel(), "gated_add_norm: out shape");
+  const int64_t rows = residual.size(0), d = residual.size(1);
+  TORCH_CHECK(w.numel() == d && bias.numel() == d, "gated_add_norm: w, bias [d]");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == rows && g_col >= 0 && g_col + d <= proj.size(1),
+              "gated_add_norm: gate columns");
+  const int yt = any_dt(y, rows * d, "y");
+  const bool v = vec8(proj, g_col, d);
+  check(k8sllm_hy_gated_add_norm(out.data_ptr(), residual.data_ptr<float>(), y.data_ptr(), yt,
+                                 (const char*)proj.data_ptr() + g_col * proj.element_size(), proj.stride(0),
+                                 bias.data_ptr<float>(), (float)mult, w.data_ptr<float>(), rows, (int)d, (float)eps, one_plus,
+                                 v, f, cur()),
+        "gated_add_norm");
+}
+
+// out [rows, f] = act(proj[:, col : col + f]) * proj[:, col + f : col + 2f]; kind 1 tanh GELU, 3 SiLU
+void glu(Tensor out, Tensor proj, int64_t col, int64_t kind) {
+  const int f = act(proj, "proj");
+  same(out, f, "out");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && out.dim() == 2 && out.is_contiguous() && out.size(0) == proj.size(0),
+              "glu: layouts");
+  const int64_t n = out.size(1);
+  TORCH_CHECK(col >= 0 && col + 2 * n <= proj.size(1) && (kind == 1 || kind == 3), "glu: columns / kind");
+  check(k8sllm_hy_glu(out.data_ptr(), (const char*)proj.data_ptr() + col * proj.element_size(), proj.stride(0), proj.size(0),
+                      (int)n, (int)kind, vec8(proj, col, n), f, cur()),
+        "glu");
+}
+
+// out [rows, n] = act(proj[:, col : col + n]); kind 0 erf GELU, 1 tanh GELU, 3 SiLU
+void activation_cols(Tensor out, Tensor proj, int64_t col, int64_t kind) {
+  const int f = act(proj, "proj");
+  same(out, f, "out");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && out.dim() == 2 && out.is_contiguous() && out.size(0) == proj.size(0),
+              "activation_cols: layouts");
+  const int64_t n = out.size(1);
+  TORCH_CHECK(col >= 0 && col + n <= proj.size(1) && (kind == 0 || kind == 1 || kind == 3), "activation_cols: columns / kind");
+  check(k8sllm_hy_activation_cols(out.data_ptr(), (const char*)proj.data_ptr() + col * proj.element_size(), proj.stride(0),
+                                  proj.size(0), (int)n, (int)kind, vec8(proj, col, n), f, cur()),
+        "activation_cols");
+}
+
+// x [rows, n] *= sigmoid(proj[:, col : col + n])
+void sigmoid_gate(Tensor x, Tensor proj, int64_t col) {
+  const int f = act(x, "x");
+  same(proj, f, "gate");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == x.size(0),
+              "sigmoid_gate: layouts");
+  const int64_t n = x.size(1);
+  TORCH_CHECK(col >= 0 && col + n <= proj.size(1), "sigmoid_gate: columns");
+  check(k8sllm_hy_sigmoid_gate(x.data_ptr(), (const char*)proj.data_ptr() + col * proj.element_size(), proj.stride(0),
+                               x.size(0), (int)n, vec8(proj, col, n), f, cur()),
+        "sigmoid_gate");
+}
+
+void softcap(Tensor x, double cap) {
+  f32c(x, "logits");
+  TORCH_CHECK(cap > 0, "softcap: cap > 0");
+  check(k8sllm_hy_softcap(x.data_ptr<float>(), x.numel(), (float)cap, cur()), "softcap");
 }
 
 void swiglu(Tensor out, Tensor gu) {
@@ -279,29 +365,79 @@ void conv_silu(Tensor out, Tensor proj, int64_t col0, Tensor cw, Tensor cb, Tens
         "conv_silu");
 }
 
-void ssm_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_col, Tensor dt_bias, Tensor a_log, Tensor d_skip,
+// decay given: the fixed-decay recurrence (dt = 1, no skip term); proj, dt_bias, a_log, d_skip are then not read
+void ssm_scan(Tensor y, Tensor xbc, OptT proj, int64_t dt_col, OptT dt_bias, OptT a_log, OptT d_skip, OptT decay,
               Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t nh, int64_t P, int64_t N, int64_t G,
               int64_t mode) {
   const int f = act(xbc, "xbc");
-  same(proj, f, "proj");
   f32c(y, "y");
-  f32c(dt_bias, "dt_bias");
-  f32c(a_log, "A_log");
-  f32c(d_skip, "D");
   f32c(state, "ssm_state");
   segs(cu, ctx, slot);
   const int64_t T = xbc.size(0);
   TORCH_CHECK(xbc.dim() == 2 && xbc.is_contiguous() && xbc.size(1) == nh * P + 2 * G * N, "xbc [T, nh*P + 2*G*N]");
-  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T && dt_col >= 0 && dt_col + nh <= proj.size(1),
-              "proj dt columns");
-  TORCH_CHECK(y.numel() == T * nh * P && dt_bias.numel() == nh && a_log.numel() == nh && d_skip.numel() == nh, "ssm sizes");
+  const void* pp = nullptr;
+  long pstride = 0;
+  const float *bp = nullptr, *ap = nullptr, *dp = nullptr, *cp = nullptr;
+  if (decay.has_value()) {
+    f32c(*decay, "decay");
+    TORCH_CHECK(decay->numel() == nh, "decay [heads]");
+    cp = decay->data_ptr<float>();
+  } else {
+    TORCH_CHECK(proj.has_value() && dt_bias.has_value() && a_log.has_value() && d_skip.has_value(), "ssm: dt inputs");
+    same(*proj, f, "proj");
+    f32c(*dt_bias, "dt_bias");
+    f32c(*a_log, "A_log");
+    f32c(*d_skip, "D");
+    TORCH_CHECK(proj->dim() == 2 && proj->stride(1) == 1 && proj->size(0) == T && dt_col >= 0 && dt_col + nh <= proj->size(1),
+                "proj dt columns");
+    TORCH_CHECK(dt_bias->numel() == nh && a_log->numel() == nh && d_skip->numel() == nh, "ssm sizes");
+    pp = proj->data_ptr();
+    pstride = proj->stride(0);
+    bp = dt_bias->data_ptr<float>();
+    ap = a_log->data_ptr<float>();
+    dp = d_skip->data_ptr<float>();
+  }
+  TORCH_CHECK(y.numel() == T * nh * P, "ssm: y [T, nh*P]");
   TORCH_CHECK(state.dim() == 4 && state.size(1) == nh && state.size(2) == N && state.size(3) == P, "ssm_state [slots, nh, N, P]");
   TORCH_CHECK(G >= 1 && nh % G == 0 && N <= 256, "ssm: groups / state size (<= 256)");
-  check(k8sllm_hy_ssm_scan(y.data_ptr<float>(), xbc.data_ptr(), proj.data_ptr(), proj.stride(0), (int)dt_col,
-                           dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), d_skip.data_ptr<float>(),
+  check(k8sllm_hy_ssm_scan(y.data_ptr<float>(), xbc.data_ptr(), pp, pstride, (int)dt_col, bp, ap, dp, cp,
                            state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
                            (int)ctx.numel(), T, (int)nh, (int)P, (int)N, (int)G, f, (int)mode, cur()),
         "ssm_scan");
+}
+
+// In place on the fused rows [T, Hq*dk | G*dk | G*dv | ...]: rotary positions on the first 2 * len(freq)
+// entries of every q / k head (pairs: entry 2i with 2i + 1, else i with i + len(freq)), q heads times
+// q_scale [Hq] (optional), k and v to the pages.
+void rotary_cache(Tensor qkv, int64_t Hq, int64_t G, int64_t dk, int64_t dv, Tensor positions, Tensor freq, bool pairs,
+                  OptT q_scale, OptT k_cache, OptT v_cache, OptT slots) {
+  const int f = act(qkv, "qkv");
+  f32c(freq, "freq");
+  i32c(positions, "positions");
+  const int64_t nq = Hq * dk, nk = G * dk, nv = G * dv, T = qkv.size(0);
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= nq + nk + nv, "qkv [T, Hq*dk + G*dk + G*dv (+ more)]");
+  TORCH_CHECK(Hq >= 1 && G >= 1 && positions.numel() >= T && 2 * freq.numel() <= dk, "rotary_cache: heads / positions / freq");
+  const float* qs = nullptr;
+  if (q_scale.has_value()) {
+    f32c(*q_scale, "q_scale");
+    TORCH_CHECK(q_scale->numel() == Hq, "q_scale [Hq]");
+    qs = q_scale->data_ptr<float>();
+  }
+  void *kc = nullptr, *vc = nullptr;
+  const int* sp = nullptr;
+  if (k_cache.has_value()) {
+    TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
+    pages(*k_cache, f, nk, "k_cache");
+    vpages(*v_cache, *k_cache, f, G, dv);
+    sp = iptr(slots, "slot_mapping");
+    TORCH_CHECK(slots->numel() >= T, "slot_mapping [T]");
+    kc = k_cache->data_ptr();
+    vc = v_cache->data_ptr();
+  }
+  check(k8sllm_hy_rotary_cache(qkv.data_ptr(), qkv.stride(0), T, (int)Hq, (int)G, (int)dk, (int)dv, positions.data_ptr<int>(),
+                               freq.data_ptr<float>(), (int)freq.numel(), pairs, qs, kc, vc, sp,
+                               k_cache.has_value() ? (int)k_cache->size(1) : 16, f, cur()),
+        "rotary_cache");
 }
 
 void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, OptT bias, int64_t E, int64_t K,
@@ -429,12 +565,12 @@ void depth_mix(Tensor stack, int64_t n, OptT addend, Tensor coef) {
 void activation(Tensor out, Tensor x, int64_t kind, double a, double b) {
   const int f = act(x, "x");
   same(out, f, "out");
-  TORCH_CHECK(x.is_contiguous() && out.is_contiguous() && out.numel() == x.numel() && kind >= 0 && kind <= 2, "activation: shapes / kind");
+  TORCH_CHECK(x.is_contiguous() && out.is_contiguous() && out.numel() == x.numel() && kind >= 0 && kind <= 3, "activation: shapes / kind");
   check(k8sllm_hy_activation(out.data_ptr(), x.data_ptr(), x.numel(), (int)kind, (float)a, (float)b, f, cur()), "activation");
 }
 
 void latent_prep(Tensor proj, int64_t Q, int64_t R, int64_t dr, Tensor qw, OptT kw, double eps, Tensor positions,
-                 Tensor freq, OptT k_cache, OptT v_cache, OptT slots) {
+                 Tensor freq, OptT k_cache, OptT v_cache, OptT slots, bool pairs) {
   const int f = act(proj, "proj");
   f32c(qw, "dq.norm");
   f32c(freq, "freq");
@@ -465,12 +601,13 @@ void latent_prep(Tensor proj, int64_t Q, int64_t R, int64_t dr, Tensor qw, OptT 
     }
   }
   check(k8sllm_hy_latent_prep(proj.data_ptr(), proj.stride(0), T, (int)Q, (int)R, (int)dr, qw.data_ptr<float>(), kwp,
-                              (float)eps, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), kc, pitch, vc,
-                              sp, bs, f, cur()),
+                              (float)eps, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), pairs, kc, pitch,
+                              vc, sp, bs, f, cur()),
         "latent_prep");
 }
 
-void latent_queries(Tensor out, Tensor q, Tensor q_lat, int64_t H, int64_t dn, int64_t dr, Tensor positions, Tensor freq) {
+void latent_queries(Tensor out, Tensor q, Tensor q_lat, int64_t H, int64_t dn, int64_t dr, Tensor positions, Tensor freq,
+                    bool pairs) {
   const int f = act(q, "q");
   same(out, f, "out");
   same(q_lat, f, "q_lat");
@@ -485,7 +622,7 @@ void latent_queries(Tensor out, Tensor q, Tensor q_lat, int64_t H, int64_t dn, i
               "latent_queries: out [T, H * pitch] / positions / freq");
   check(k8sllm_hy_latent_queries(out.data_ptr(), q.data_ptr(), q.stride(0), q_lat.data_ptr(), T, (int)H, (int)dn, (int)dr,
                                  (int)R, (int)(out.size(1) / H), positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(),
-                                 f, cur()),
+                                 pairs, f, cur()),
         "latent_queries");
 }
 
@@ -533,6 +670,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_norm", &add_norm);
   m.def("gated_group_norm", &gated_group_norm);
   m.def("swiglu", &swiglu);
+  m.def("gated_add_norm", &gated_add_norm);
+  m.def("glu", &glu);
+  m.def("activation_cols", &activation_cols);
+  m.def("sigmoid_gate", &sigmoid_gate);
+  m.def("softcap", &softcap);
+  m.def("rotary_cache", &rotary_cache);
   m.def("qk_norm_cache", &qk_norm_cache);
   m.def("window_attention_prefill", &window_attention_prefill);
   m.def("window_attention_decode", &window_attention_decode);

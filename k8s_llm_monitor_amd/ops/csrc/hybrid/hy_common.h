@@ -77,6 +77,7 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 }
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
 
 // the segment that holds row r: largest s with cu[s] <= r (cu has S + 1 entries, cu[0] = 0)
 __device__ __forceinline__ int find_segment(const int* __restrict__ cu, int S, int r) {

@@ -6,8 +6,9 @@
 //   latent_queries  per head [q_lat (unrotated query times the key expansion) | rotated query part |
 //                   zeros up to the same pitch]
 //   latent_attention  the matrix-core attention over those pages (bf16), prompt chunks and decoding
-// Rotation: entries i and i + n/2 of the first 2 * nf entries (nf frequencies, freq[i] given in fp32)
-// turn by the angle position * freq[i]; angles, sine and cosine are fp32.
+// Rotation: entries i and i + nf of the first 2 * nf entries (nf frequencies, freq[i] given in fp32)
+// turn by the angle position * freq[i] - or, pairs == 1, entries 2i and 2i + 1; angles, sine and cosine
+// are fp32.
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -16,7 +17,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ proj, long stride, int Q, int R, int dr,
                                                           const float* __restrict__ qw, const float* __restrict__ kw,
                                                           float eps, const int* __restrict__ positions,
-                                                          const float* __restrict__ freq, int nf,
+                                                          const float* __restrict__ freq, int nf, int pairs,
                                                           T* __restrict__ k_cache, int kw_pitch,
                                                           T* __restrict__ v_cache,
                                                           const int* __restrict__ slots, int bs) {
@@ -51,15 +52,16 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ proj, 
   T* kr = row + Q + R;
   const float pos = (float)positions[t];
   for (int i = threadIdx.x; i < dr; i += 256) {
-    if (i < nf) {  // this thread owns the pair (i, i + nf)
+    if (i < nf) {  // this thread owns the pair (i, i + nf), or (2i, 2i + 1)
+      const int a = pairs ? 2 * i : i, b = pairs ? 2 * i + 1 : i + nf;
       float sn, cs;
       sincosf(pos * freq[i], &sn, &cs);
-      const float u = ldf(kr + i), v = ldf(kr + i + nf);
-      stf(kr + i, u * cs - v * sn);
-      stf(kr + i + nf, v * cs + u * sn);
+      const float u = ldf(kr + a), v = ldf(kr + b);
+      stf(kr + a, u * cs - v * sn);
+      stf(kr + b, v * cs + u * sn);
       if (kp != nullptr) {
-        kp[R + i] = kr[i];
-        kp[R + i + nf] = kr[i + nf];
+        kp[R + a] = kr[a];
+        kp[R + b] = kr[b];
       }
     } else if (i >= 2 * nf && kp != nullptr) {
       kp[R + i] = kr[i];
@@ -71,7 +73,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out, const T* __restrict__ q, long q_stride,
                                                              const T* __restrict__ q_lat, long T_rows, int H, int dn,
                                                              int dr, int R, int w, const int* __restrict__ positions,
-                                                             const float* __restrict__ freq, int nf) {
+                                                             const float* __restrict__ freq, int nf, int pairs) {
   const long t = blockIdx.x;
   const float pos = (float)positions[t];
   T* o = out + t * (long)H * w;
@@ -91,11 +93,12 @@ __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out
       o[c] = qr[i];
       continue;
     }
-    const int f = i < nf ? i : i - nf;
+    const int f = pairs ? i >> 1 : (i < nf ? i : i - nf);
+    const bool lead = pairs ? !(i & 1) : i < nf;  // the pair's first entry
     float sn, cs;
     sincosf(pos * freq[f], &sn, &cs);
-    const float u = ldf(qr + f), v = ldf(qr + f + nf);
-    stf(o + c, i < nf ? u * cs - v * sn : v * cs + u * sn);
+    const float u = ldf(qr + (pairs ? 2 * f : f)), v = ldf(qr + (pairs ? 2 * f + 1 : f + nf));
+    stf(o + c, lead ? u * cs - v * sn : v * cs + u * sn);
   }
 }
 
@@ -567,29 +570,30 @@ using namespace k8sllm;
 extern "C" {
 
 int k8sllm_hy_latent_prep(void* proj, long stride, long T, int Q, int R, int dr, const float* qw, const float* kw,
-                          float eps, const int* positions, const float* freq, int nf, void* k_cache, int kw_pitch,
-                          void* v_cache, const int* slots, int bs, int f32, hipStream_t s) {
+                          float eps, const int* positions, const float* freq, int nf, int pairs, void* k_cache,
+                          int kw_pitch, void* v_cache, const int* slots, int bs, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (2 * nf > dr || (k_cache != nullptr && kw_pitch < R + dr)) return -1;
   if (f32)
     hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(T), dim3(256), 0, s, (float*)proj, stride, Q, R, dr, qw, kw, eps,
-                       positions, freq, nf, (float*)k_cache, kw_pitch, (float*)v_cache, slots, bs);
+                       positions, freq, nf, pairs, (float*)k_cache, kw_pitch, (float*)v_cache, slots, bs);
   else
     hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)proj, stride, Q, R, dr, qw, kw,
-                       eps, positions, freq, nf, (bf16_t*)k_cache, kw_pitch, (bf16_t*)v_cache, slots, bs);
+                       eps, positions, freq, nf, pairs, (bf16_t*)k_cache, kw_pitch, (bf16_t*)v_cache, slots, bs);
   return (int)hipGetLastError();
 }
 
 int k8sllm_hy_latent_queries(void* out, const void* q, long q_stride, const void* q_lat, long T, int H, int dn, int dr,
-                             int R, int w, const int* positions, const float* freq, int nf, int f32, hipStream_t s) {
+                             int R, int w, const int* positions, const float* freq, int nf, int pairs, int f32,
+                             hipStream_t s) {
   if (T <= 0) return 0;
   if (2 * nf > dr || w < R + dr) return -1;
   if (f32)
     hipLaunchKernelGGL(latent_queries_kernel<float>, dim3(T), dim3(256), 0, s, (float*)out, (const float*)q, q_stride,
-                       (const float*)q_lat, T, H, dn, dr, R, w, positions, freq, nf);
+                       (const float*)q_lat, T, H, dn, dr, R, w, positions, freq, nf, pairs);
   else
     hipLaunchKernelGGL(latent_queries_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)q,
-                       q_stride, (const bf16_t*)q_lat, T, H, dn, dr, R, w, positions, freq, nf);
+                       q_stride, (const bf16_t*)q_lat, T, H, dn, dr, R, w, positions, freq, nf, pairs);
   return (int)hipGetLastError();
 }
 // Matrix-core latent attention (bf16): rows = T tokens, each at the position its segment (cu / ctx,

@@ -4,7 +4,10 @@
 //                    sequence's conv state slot (zeros for a sequence that starts in this step)
 //   conv_state_step  advances each segment's conv state slot to the segment's end
 //   ssm_scan         S <- exp(-exp(A_log) dt) S + dt B x^T;  y = S^T C + D x, token by token per
-//                    segment; the state slot [nh][N][P] is read at the start, written at the end
+//                    segment; the state slot [nh][N][P] is read at the start, written at the end.
+//                    With a table of fixed decays per head (``decay``) the same scan is the linear
+//                    attention recurrence S <- decay S + k v^T, y = S^T q (dt = 1, no skip term; B, C, x
+//                    are k, q, v)
 // A segment is one sequence's rows of this step: cu[s] .. cu[s+1], ctx[s] tokens already in its
 // state (0: starts from zero), slot[s] its state slot (< 0: skipped).
 #include "hy_common.h"
@@ -136,7 +139,8 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
                                                        const T* __restrict__ proj, long p_stride, int dt_col,
                                                        const float* __restrict__ dt_bias,
                                                        const float* __restrict__ a_log,
-                                                       const float* __restrict__ d_skip, float* __restrict__ state,
+                                                       const float* __restrict__ d_skip,
+                                                       const float* __restrict__ decay, float* __restrict__ state,
                                                        const int* __restrict__ cu, const int* __restrict__ ctx,
                                                        const int* __restrict__ slot, int nh, int P, int N, int G) {
   constexpr int TB = 16;
@@ -170,7 +174,9 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
   const bool carried = ctx[s] > 0;
 #pragma unroll
   for (int i = 0; i < NPT; ++i) S[i] = (carried && live && n0 + i < N) ? sp[(long)(n0 + i) * P] : 0.f;
-  const float A = expf(a_log[h]), Dh = d_skip[h], bias = dt_bias[h];
+  const bool fixed = decay != nullptr;  // fixed decay per head: dt = 1, no skip term
+  const float A = fixed ? 0.f : expf(a_log[h]), Dh = fixed ? 0.f : d_skip[h], bias = fixed ? 0.f : dt_bias[h];
+  const float dfix = fixed ? decay[h] : 0.f;
   for (int tb = t0; tb < t1; tb += TB) {
     const int nt = min(TB, t1 - tb);
     __syncthreads();  // the previous tile is consumed (and the zero fill is done)
@@ -189,10 +195,15 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
       xs[tt][pp] = pg < P ? ldf(xbc + (long)(tb + tt) * C + (long)h * P + pg) : 0.f;
     }
     if (threadIdx.x < nt) {
-      const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
-      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-      dts[threadIdx.x] = dt;
-      dAs[threadIdx.x] = expf(-A * dt);
+      if (fixed) {
+        dts[threadIdx.x] = 1.f;
+        dAs[threadIdx.x] = dfix;
+      } else {
+        const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
+        const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+        dts[threadIdx.x] = dt;
+        dAs[threadIdx.x] = expf(-A * dt);
+      }
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
@@ -234,6 +245,7 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
                                                             const float* __restrict__ dt_bias,
                                                             const float* __restrict__ a_log,
                                                             const float* __restrict__ d_skip,
+                                                            const float* __restrict__ decay,
                                                             float* __restrict__ state, const int* __restrict__ cu,
                                                             const int* __restrict__ ctx, const int* __restrict__ slot,
                                                             int nh, int P, int N, int G) {
@@ -268,7 +280,9 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
   const bool carried = ctx[s] > 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) S[i] = (carried && live && n0 + i < N) ? sp[(long)(n0 + i) * P] : 0.f;
-  const float A = expf(a_log[h]), Dh = d_skip[h], bias = dt_bias[h];
+  const bool fixed = decay != nullptr;  // fixed decay per head: dt = 1, no skip term
+  const float A = fixed ? 0.f : expf(a_log[h]), Dh = fixed ? 0.f : d_skip[h], bias = fixed ? 0.f : dt_bias[h];
+  const float dfix = fixed ? decay[h] : 0.f;
   const int boff = n0 + (n0 >> 6) * 4;
   // a thread stages the same elements of every tile: their token, LDS offset and offset from the
   // tile's first row are computed once (the division by N is ~40 instructions)
@@ -300,10 +314,15 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
       xs[tt][pp] = pg < P ? ldf(xbc + (long)(tb + tt) * C + (long)h * P + pg) : 0.f;
     }
     if (threadIdx.x < nt) {
-      const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
-      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-      dts[threadIdx.x] = dt;
-      dAs[threadIdx.x] = expf(-A * dt);
+      if (fixed) {
+        dts[threadIdx.x] = 1.f;
+        dAs[threadIdx.x] = dfix;
+      } else {
+        const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
+        const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+        dts[threadIdx.x] = dt;
+        dAs[threadIdx.x] = expf(-A * dt);
+      }
     }
     __syncthreads();
 #pragma unroll 2
@@ -342,12 +361,12 @@ using namespace k8sllm;
 
 template <typename T>
 static int launch_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
-                       const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
+                       const float* a_log, const float* d_skip, const float* decay, float* state, const int* cu, const int* ctx,
                        const int* slot, int S, int nh, int P, int N, int G, int wide, hipStream_t s) {
   if (wide && N > 8) {  // long segments: 8 states per lane
 #define K8SLLM_WIDE(CH)                                                                                              \
   hipLaunchKernelGGL((ssm_scan_wide_kernel<T, CH>), dim3((unsigned)S, (unsigned)nh, (unsigned)((P + 256 / CH - 1) / (256 / CH))), \
-                     dim3(256), 0, s, y, (const T*)xbc, (const T*)proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, \
+                     dim3(256), 0, s, y, (const T*)xbc, (const T*)proj, p_stride, dt_col, dt_bias, a_log, d_skip, decay, state, \
                      cu, ctx, slot, nh, P, N, G)
     if (N <= 16) K8SLLM_WIDE(2);
     else if (N <= 32) K8SLLM_WIDE(4);
@@ -361,7 +380,7 @@ static int launch_scan(float* y, const void* xbc, const void* proj, long p_strid
   const dim3 grid((unsigned)S, (unsigned)nh, (unsigned)((P + 63) / 64));
 #define K8SLLM_SCAN(NPT)                                                                                              \
   hipLaunchKernelGGL((ssm_scan_kernel<T, NPT>), grid, dim3(256), 0, s, y, (const T*)xbc, (const T*)proj, p_stride,    \
-                     dt_col, dt_bias, a_log, d_skip, state, cu, ctx, slot, nh, P, N, G)
+                     dt_col, dt_bias, a_log, d_skip, decay, state, cu, ctx, slot, nh, P, N, G)
   if (N <= 16) K8SLLM_SCAN(4);
   else if (N <= 32) K8SLLM_SCAN(8);
   else if (N <= 64) K8SLLM_SCAN(16);
@@ -407,15 +426,16 @@ int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int 
 }
 
 int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
-                       const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
+                       const float* a_log, const float* d_skip, const float* decay, float* state, const int* cu, const int* ctx,
                        const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode, hipStream_t s) {
   if (S <= 0) return 0;
   if (G < 1 || nh % G) return -1;
   // mode 0: by the step's mean segment length (prompts: the thin mapping); 1 / 2: forced (tests)
   const int wide = mode == 2 || (mode == 0 && T >= 32L * S);
-  return f32 ? launch_scan<float>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, cu, ctx, slot, S, nh,
-                                  P, N, G, wide, s)
-             : launch_scan<bf16_t>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, cu, ctx, slot, S,
-                                   nh, P, N, G, wide, s);
+  if (decay == nullptr && (proj == nullptr || dt_bias == nullptr || a_log == nullptr || d_skip == nullptr)) return -1;
+  return f32 ? launch_scan<float>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, decay, state, cu, ctx, slot,
+                                  S, nh, P, N, G, wide, s)
+             : launch_scan<bf16_t>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, decay, state, cu, ctx, slot,
+                                   S, nh, P, N, G, wide, s);
 }
 }

@@ -6,7 +6,12 @@
 //   norm_shift        h[t] = x[t] / rms(x[t]) * w;  out[t] = h[t] + (h[t-1] - h[t]) * mu, the row before
 //                     a segment from the sequence's state slot; shift_state advances the slots
 //   depth_mix         stack[n] += addend;  stack[n+1] = sum_j coef[j] * stack[j], j = 0 .. n
-//   activation        erf GELU, tanh GELU or xIELU, elementwise in fp32
+//   activation        erf GELU, tanh GELU, xIELU or SiLU, elementwise in fp32 (also over a column range)
+//   gated_add_norm    residual += mult * y * sigmoid(gate + bias);  out = residual / rms(residual) * w
+//   glu               out = act(gu[:, :f]) * gu[:, f:2f]           (rows may be wider than 2f)
+//   norm_gate         out = y / rms(y) * w * sigmoid(z)            (y fp32)
+//   sigmoid_gate      x *= sigmoid(z), in place
+//   softcap           x = cap * tanh(x / cap), in place (fp32 logits)
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -96,13 +101,21 @@ template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(T* __restrict__ out, const float* __restrict__ y,
                                                                const T* __restrict__ z, long z_stride,
                                                                const float* __restrict__ w, int n, int groups,
-                                                               float eps) {
+                                                               float eps, int after) {
   __shared__ float red[4];
   const long row = blockIdx.x;
   const int g = blockIdx.y, gs = n / groups;
   const float* yr = y + row * n + (long)g * gs;
   const T* zr = z + row * z_stride + (long)g * gs;
   float ss = 0.f;
+  if (after) {  // the norm first, then a sigmoid gate
+    for (int c = threadIdx.x; c < gs; c += 256) ss += yr[c] * yr[c];
+    ss = block_sum<256>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int c = threadIdx.x; c < gs; c += 256)
+      stf(out + row * n + (long)g * gs + c, yr[c] * inv * w[(long)g * gs + c] * sigmoid_f(ldf(zr + c)));
+    return;
+  }
   for (int c = threadIdx.x; c < gs; c += 256) {
     const float v = yr[c] * silu_f(ldf(zr + c));
     ss += v * v;
@@ -113,6 +126,57 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(T* __restrict__ o
     const float v = yr[c] * silu_f(ldf(zr + c));
     stf(out + row * n + (long)g * gs + c, v * inv * w[(long)g * gs + c]);
   }
+}
+
+// residual += mult * y * sigmoid(gate + bias), then the RMSNorm of the new residual times w.  y: any
+// float dtype, contiguous; gate: activation dtype, rows g_stride apart (a column range of a wider
+// projection).  Sum, sigmoid and norm are fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_add_norm_kernel(T* __restrict__ out, float* __restrict__ residual,
+                                                             const void* __restrict__ y, int yt,
+                                                             const T* __restrict__ gate, long g_stride,
+                                                             const float* __restrict__ bias, float mult,
+                                                             const float* __restrict__ w, int d, float eps,
+                                                             int one_plus, int vec) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float* r = residual + row * d;
+  const T* gr = gate + row * g_stride;
+  float ss = 0.f;
+  if (vec) {  // d, the gate's row stride and column offset are multiples of 8
+    for (int c = threadIdx.x * 8; c < d; c += 2048) {
+      float x[8], a[8], g[8], b[8];
+      load8(r + c, x);
+      load8_any(y, yt, row * d + c, a);
+      load8(gr + c, g);
+      load8(bias + c, b);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] += mult * a[i] * sigmoid_f(g[i] + b[i]);
+        ss += x[i] * x[i];
+      }
+      store8(r + c, x);
+    }
+    ss = block_sum<256>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int c = threadIdx.x * 8; c < d; c += 2048) {  // each thread re-reads what it wrote
+      float x[8], g[8];
+      load8(r + c, x);
+      load8(w + c, g);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] *= inv * (one_plus ? 1.f + g[i] : g[i]);
+      store8(out + row * d + c, x);
+    }
+    return;
+  }
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float x = r[c] + mult * ld_any(y, yt, row * d + c) * sigmoid_f(ldf(gr + c) + bias[c]);
+    r[c] = x;
+    ss += x * x;
+  }
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += 256) stf(out + row * d + c, r[c] * inv * (one_plus ? 1.f + w[c] : w[c]));
 }
 
 template <typename T>
@@ -231,12 +295,82 @@ __global__ __launch_bounds__(256) void depth_mix_scalar_kernel(float* __restrict
   stack[(long)(n + 1) * plane + i] = acc + coef[n] * top;
 }
 
-// KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below)
+// KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below), 3: SiLU
 template <int KIND>
 __device__ __forceinline__ float act_f(float z, float a, float b) {
   if (KIND == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
   if (KIND == 1) return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+  if (KIND == 3) return z / (1.f + expf(-z));
   return z > 0.f ? a * z * z + 0.5f * z : b * (expm1f(z) - z) + 0.5f * z;
+}
+
+// out [rows, n] (contiguous) = act(x[:, 0:n]) where x's rows are x_stride apart; 8 columns per thread
+// where n, the stride and the column offset are multiples of 8 (vec)
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void activation_cols_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                                              long x_stride, long rows, int n, int vec) {
+  const int per = vec ? n / 8 : n;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * per) return;
+  const long r = i / per;
+  const int c = (int)(i - r * per);
+  if (vec) {
+    float v[8];
+    load8(x + r * x_stride + 8 * c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = act_f<KIND>(v[k], 0.f, 0.f);
+    store8(out + r * n + 8 * c, v);
+    return;
+  }
+  stf(out + r * n + c, act_f<KIND>(ldf(x + r * x_stride + c), 0.f, 0.f));
+}
+
+// out [rows, f] = act(gu[:, 0:f]) * gu[:, f:2f], gu's rows g_stride apart
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void glu_kernel(T* __restrict__ out, const T* __restrict__ gu, long g_stride,
+                                                  long rows, int f, int vec) {
+  const int per = vec ? f / 8 : f;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * per) return;
+  const long r = i / per;
+  const int c = (int)(i - r * per);
+  const T* g = gu + r * g_stride;
+  if (vec) {
+    float a[8], u[8];
+    load8(g + 8 * c, a);
+    load8(g + f + 8 * c, u);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] = act_f<KIND>(a[k], 0.f, 0.f) * u[k];
+    store8(out + r * f + 8 * c, a);
+    return;
+  }
+  stf(out + r * f + c, act_f<KIND>(ldf(g + c), 0.f, 0.f) * ldf(g + f + c));
+}
+
+// x [rows, n] (contiguous) *= sigmoid(z[:, 0:n]), z's rows z_stride apart
+template <typename T>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(T* __restrict__ x, const T* __restrict__ z, long z_stride,
+                                                           long rows, int n, int vec) {
+  const int per = vec ? n / 8 : n;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * per) return;
+  const long r = i / per;
+  const int c = (int)(i - r * per);
+  if (vec) {
+    float a[8], g[8];
+    load8(x + r * n + 8 * c, a);
+    load8(z + r * z_stride + 8 * c, g);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] *= sigmoid_f(g[k]);
+    store8(x + r * n + 8 * c, a);
+    return;
+  }
+  stf(x + r * n + c, ldf(x + r * n + c) * sigmoid_f(ldf(z + r * z_stride + c)));
+}
+
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, long n, float cap) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] = cap * tanhf(x[i] / cap);
 }
 
 template <typename T, int KIND>
@@ -287,16 +421,80 @@ int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const
   return (int)hipGetLastError();
 }
 
+// after 0: group_rms_norm(y * silu(z)) * w;  1: group_rms_norm(y) * w * sigmoid(z)
 int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_stride, const float* w, long rows,
-                               int n, int groups, float eps, int f32, hipStream_t s) {
+                               int n, int groups, float eps, int after, int f32, hipStream_t s) {
   if (rows <= 0) return 0;
   if (groups < 1 || n % groups) return -1;
   if (f32)
     hipLaunchKernelGGL(gated_group_norm_kernel<float>, dim3(rows, groups), dim3(256), 0, s, (float*)out, y,
-                       (const float*)z, z_stride, w, n, groups, eps);
+                       (const float*)z, z_stride, w, n, groups, eps, after);
   else
     hipLaunchKernelGGL(gated_group_norm_kernel<bf16_t>, dim3(rows, groups), dim3(256), 0, s, (bf16_t*)out, y,
-                       (const bf16_t*)z, z_stride, w, n, groups, eps);
+                       (const bf16_t*)z, z_stride, w, n, groups, eps, after);
+  return (int)hipGetLastError();
+}
+
+// yt: 1 = bf16, 2 = fp32; vec: 8-wide accesses are aligned (checked by the caller)
+int k8sllm_hy_gated_add_norm(void* out, float* residual, const void* y, int yt, const void* gate, long g_stride,
+                             const float* bias, float mult, const float* w, long rows, int d, float eps, int one_plus,
+                             int vec, int f32, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (f32)
+    hipLaunchKernelGGL(gated_add_norm_kernel<float>, dim3(rows), dim3(256), 0, s, (float*)out, residual, y, yt,
+                       (const float*)gate, g_stride, bias, mult, w, d, eps, one_plus, vec);
+  else
+    hipLaunchKernelGGL(gated_add_norm_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, (bf16_t*)out, residual, y, yt,
+                       (const bf16_t*)gate, g_stride, bias, mult, w, d, eps, one_plus, vec);
+  return (int)hipGetLastError();
+}
+
+// kind: 1 tanh GELU, 3 SiLU
+int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, int vec, int f32,
+                  hipStream_t s) {
+  const long n = rows * (vec ? f / 8 : f);
+  if (n <= 0) return 0;
+  const dim3 g((unsigned)((n + 255) / 256));
+#define K8SLLM_GLU(T, K) hipLaunchKernelGGL((glu_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)gu, g_stride, rows, f, vec)
+  if (f32) {
+    if (kind == 1) K8SLLM_GLU(float, 1); else if (kind == 3) K8SLLM_GLU(float, 3); else return -1;
+  } else {
+    if (kind == 1) K8SLLM_GLU(bf16_t, 1); else if (kind == 3) K8SLLM_GLU(bf16_t, 3); else return -1;
+  }
+#undef K8SLLM_GLU
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_activation_cols(void* out, const void* x, long x_stride, long rows, int n, int kind, int vec, int f32,
+                              hipStream_t s) {
+  const long tot = rows * (vec ? n / 8 : n);
+  if (tot <= 0) return 0;
+  const dim3 g((unsigned)((tot + 255) / 256));
+#define K8SLLM_AC(T, K) hipLaunchKernelGGL((activation_cols_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)x, x_stride, rows, n, vec)
+  if (f32) {
+    if (kind == 0) K8SLLM_AC(float, 0); else if (kind == 1) K8SLLM_AC(float, 1); else if (kind == 3) K8SLLM_AC(float, 3); else return -1;
+  } else {
+    if (kind == 0) K8SLLM_AC(bf16_t, 0); else if (kind == 1) K8SLLM_AC(bf16_t, 1); else if (kind == 3) K8SLLM_AC(bf16_t, 3); else return -1;
+  }
+#undef K8SLLM_AC
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_sigmoid_gate(void* x, const void* z, long z_stride, long rows, int n, int vec, int f32, hipStream_t s) {
+  const long tot = rows * (vec ? n / 8 : n);
+  if (tot <= 0) return 0;
+  const dim3 g((unsigned)((tot + 255) / 256));
+  if (f32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, g, dim3(256), 0, s, (float*)x, (const float*)z, z_stride, rows, n, vec);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, g, dim3(256), 0, s, (bf16_t*)x, (const bf16_t*)z, z_stride, rows, n, vec);
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_softcap(float* x, long n, float cap, hipStream_t s) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return -1;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, cap);
   return (int)hipGetLastError();
 }
 
@@ -345,9 +543,9 @@ int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, fl
   const dim3 g((unsigned)((n + 2047) / 2048));
 #define K8SLLM_ACT(T, K) hipLaunchKernelGGL((activation_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)x, n, a, b)
   if (f32) {
-    if (kind == 0) K8SLLM_ACT(float, 0); else if (kind == 1) K8SLLM_ACT(float, 1); else if (kind == 2) K8SLLM_ACT(float, 2); else return -1;
+    if (kind == 0) K8SLLM_ACT(float, 0); else if (kind == 1) K8SLLM_ACT(float, 1); else if (kind == 2) K8SLLM_ACT(float, 2); else if (kind == 3) K8SLLM_ACT(float, 3); else return -1;
   } else {
-    if (kind == 0) K8SLLM_ACT(bf16_t, 0); else if (kind == 1) K8SLLM_ACT(bf16_t, 1); else if (kind == 2) K8SLLM_ACT(bf16_t, 2); else return -1;
+    if (kind == 0) K8SLLM_ACT(bf16_t, 0); else if (kind == 1) K8SLLM_ACT(bf16_t, 1); else if (kind == 2) K8SLLM_ACT(bf16_t, 2); else if (kind == 3) K8SLLM_ACT(bf16_t, 3); else return -1;
   }
 #undef K8SLLM_ACT
   return (int)hipGetLastError();

@@ -3,7 +3,10 @@ windowed attention with a softmax sink over a paged cache, the Mamba-2 recurrenc
 convolution and per-sequence state slots, and routed experts with a biased fp32 router and a
 gated shared expert; and, for the sequential-block designs, the token-shifted norm, the depth
 average of layer results, latent (low-rank compressed) attention with rotary positions and learned
-per-head sinks, and ungated experts with a softmax-over-all router.
+per-head sinks, and ungated experts with a softmax-over-all router; and the gated residual
+(a sublayer's result times the sigmoid of a projection of its input, scaled, then the norm),
+rotary grouped-query attention with per-head temperatures, the fixed-decay linear-attention
+recurrence, gated linear units and the logit soft cap.
 
 GPU tensors run the gfx950 kernels of ``_k8sllm_hybrid`` (``ops/csrc/hybrid``; built by
 ``python -m k8s_llm_monitor_amd.ops.build --only hybrid``) for bfloat16 and float32 activations
@@ -100,6 +103,25 @@ def add_norm(residual: torch.Tensor, addends: tuple, vec: Optional[torch.Tensor]
     return out
 
 
+def gated_add_norm(residual: torch.Tensor, y: torch.Tensor, proj: torch.Tensor, g_col: int, bias: torch.Tensor,
+                   mult: float, w: torch.Tensor, eps: float, one_plus: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """Gated residual: ``residual`` (fp32 [T, d], updated in place) += ``mult * y * sigmoid(g + bias)``
+    with the gate logits ``g = proj[:, g_col : g_col + d]`` (a column range of a wider projection of
+    the sublayer's input, activation dtype) and ``bias`` [d] fp32; returns the RMSNorm of the new
+    residual times ``w`` (``one_plus``: ``1 + w``) in ``out_dtype``.  ``y`` [T, d]: any float dtype.
+    Sigmoid, product, sum and norm are fp32."""
+    d = residual.shape[1]
+    if not residual.is_cuda:
+        g = proj[:, g_col:g_col + d].float() + bias.float()
+        residual += mult * y.float() * torch.sigmoid(g)
+        h = residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+        wf = w.float()
+        return (h * (1.0 + wf if one_plus else wf)).to(out_dtype)
+    out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    native().gated_add_norm(out, residual, y.contiguous(), proj, int(g_col), bias, float(mult), w, float(eps), bool(one_plus))
+    return out
+
+
 def norm_shift(residual: torch.Tensor, addends: tuple, w: torch.Tensor, eps: float, one_plus: bool,
                mu: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
                seg_slot: torch.Tensor, out_dtype: torch.dtype, advance: bool = True,
@@ -150,27 +172,72 @@ def depth_mix(stack: torch.Tensor, n: int, addend: Optional[torch.Tensor], coef:
     return stack[n + 1]
 
 
-ACTS = {"gelu": 0, "gelu_tanh": 1, "xielu": 2}
+ACTS = {"gelu": 0, "gelu_tanh": 1, "xielu": 2, "silu": 3}
+
+
+def _act_torch(z: torch.Tensor, kind: str) -> torch.Tensor:
+    if kind == "gelu":
+        return F.gelu(z)
+    if kind == "gelu_tanh":
+        return F.gelu(z, approximate="tanh")
+    if kind == "silu":
+        return _silu(z)
+    raise ValueError(kind)
 
 
 def activation(x: torch.Tensor, kind: str, a: float = 0.0, b: float = 0.0) -> torch.Tensor:
-    """Elementwise on [T, f] rows, evaluated in fp32: ``gelu`` (erf form), ``gelu_tanh``, or
+    """Elementwise on [T, f] rows, evaluated in fp32: ``gelu`` (erf form), ``gelu_tanh``, ``silu``, or
     ``xielu`` with the two positive constants ``a``, ``b``:  z > 0: a z^2 + z / 2;  z <= 0:
     b (exp(z) - 1 - z) + z / 2."""
     if not x.is_cuda:
         z = x.float()
-        if kind == "gelu":
-            y = F.gelu(z)
-        elif kind == "gelu_tanh":
-            y = F.gelu(z, approximate="tanh")
-        elif kind == "xielu":
+        if kind == "xielu":
             y = torch.where(z > 0, a * z * z + 0.5 * z, b * (torch.expm1(z.clamp(max=0.0)) - z) + 0.5 * z)
         else:
-            raise ValueError(kind)
+            y = _act_torch(z, kind)
         return y.to(x.dtype)
     out = torch.empty_like(x)
     native().activation(out, x, ACTS[kind], float(a), float(b))
     return out
+
+
+def activation_cols(proj: torch.Tensor, col: int, n: int, kind: str) -> torch.Tensor:
+    """``act(proj[:, col : col + n])`` as a contiguous [T, n] tensor (``gelu``, ``gelu_tanh`` or
+    ``silu``, evaluated in fp32): the activation of a column range of a wider projection."""
+    if not proj.is_cuda:
+        return _act_torch(proj[:, col:col + n].float(), kind).to(proj.dtype)
+    out = torch.empty(proj.shape[0], n, dtype=proj.dtype, device=proj.device)
+    native().activation_cols(out, proj, int(col), ACTS[kind])
+    return out
+
+
+def glu(proj: torch.Tensor, col: int, f: int, kind: str) -> torch.Tensor:
+    """Gated linear unit ``act(proj[:, col : col + f]) * proj[:, col + f : col + 2 f]`` ([gate | up]
+    columns of a possibly wider projection) with ``kind`` ``gelu_tanh`` or ``silu``; fp32 arithmetic,
+    [T, f] in the activation dtype."""
+    if not proj.is_cuda:
+        return (_act_torch(proj[:, col:col + f].float(), kind) * proj[:, col + f:col + 2 * f].float()).to(proj.dtype)
+    out = torch.empty(proj.shape[0], f, dtype=proj.dtype, device=proj.device)
+    native().glu(out, proj, int(col), ACTS[kind])
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, proj: torch.Tensor, col: int) -> torch.Tensor:
+    """In place: ``x`` [T, n] *= sigmoid(proj[:, col : col + n]) (fp32 arithmetic)."""
+    n = x.shape[1]
+    if not x.is_cuda:
+        x.copy_((x.float() * torch.sigmoid(proj[:, col:col + n].float())).to(x.dtype))
+        return x
+    native().sigmoid_gate(x, proj, int(col))
+    return x
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """In place on fp32 logits: ``cap * tanh(logits / cap)``."""
+    if not logits.is_cuda:
+        return logits.copy_(cap * torch.tanh(logits / cap))
+    native().softcap(logits, float(cap))
+    return logits
 
 
 # ---------------------------------------------------------------- windowed attention with a sink
@@ -197,6 +264,34 @@ def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: fl
             v_cache.view(-1, Hkv * dv, bs)[s // bs, :, s % bs] = qkv[ok, nq + nk:]
         return
     native().qk_norm_cache(qkv, qw, kw, float(eps), Hq, Hkv, dk, dv, k_cache, v_cache, slot_mapping)
+
+
+def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positions: torch.Tensor, freq: torch.Tensor,
+                 pairs: bool, q_scale: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                 v_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> None:
+    """In place on the fused rows [T, Hq*dk | Hkv*dk | Hkv*dv | ...]: the first ``2 len(freq)`` entries
+    of every query and key head turn by the angle ``position * freq[i]`` (fp32; ``pairs``: entry 2i
+    with 2i + 1, else entry i with i + len(freq); rotary_freq); the rest of a head passes.  ``q_scale``
+    [Hq] fp32 (optional): every query head is multiplied by its number in the same pass (a per-head
+    temperature folded into the query).  Keys (turned) and values go to the paged cache at
+    ``slot_mapping`` (< 0: not written)."""
+    nq, nk, nv = Hq * dk, Hkv * dk, Hkv * dv
+    if not qkv.is_cuda:
+        T = qkv.shape[0]
+        q = _rotate(qkv[:, :nq].float().view(T, Hq, dk), positions, freq, pairs)
+        if q_scale is not None:
+            q = q * q_scale.float().view(1, Hq, 1)
+        k = _rotate(qkv[:, nq:nq + nk].float().view(T, Hkv, dk), positions, freq, pairs)
+        qkv[:, :nq] = q.reshape(T, nq).to(qkv.dtype)
+        qkv[:, nq:nq + nk] = k.reshape(T, nk).to(qkv.dtype)
+        if k_cache is not None:
+            ok = slot_mapping[:T] >= 0
+            s = slot_mapping[:T][ok].long()
+            k_cache.view(-1, nk)[s] = qkv[ok, nq:nq + nk]
+            bs = k_cache.shape[1]
+            v_cache.view(-1, nv, bs)[s // bs, :, s % bs] = qkv[ok, nq + nk:nq + nk + nv]
+        return
+    native().rotary_cache(qkv, Hq, Hkv, dk, dv, positions, freq, bool(pairs), q_scale, k_cache, v_cache, slot_mapping)
 
 
 def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sink: bool,
@@ -293,14 +388,31 @@ def _rotate_half(v: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor) -> torc
     return torch.cat([u * c - x * s, x * c + u * s, v[..., 2 * half:]], -1)
 
 
+def _rotate_pairs(v: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor) -> torch.Tensor:
+    """The same turn with entries 2i and 2i + 1 paired (i < len(freq))."""
+    nf = freq.numel()
+    a = pos[:v.shape[0]].float().view(-1, *([1] * (v.dim() - 1))) * freq.float()
+    c, s = torch.cos(a), torch.sin(a)
+    u, x = v[..., 0:2 * nf:2], v[..., 1:2 * nf:2]
+    out = v.clone()
+    out[..., 0:2 * nf:2] = u * c - x * s
+    out[..., 1:2 * nf:2] = x * c + u * s
+    return out
+
+
+def _rotate(v: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor, pairs: bool) -> torch.Tensor:
+    return _rotate_pairs(v, pos, freq) if pairs else _rotate_half(v, pos[:v.shape[0]], freq)
+
+
 def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw: torch.Tensor,
                 kw: Optional[torch.Tensor], eps: float, positions: torch.Tensor, freq: torch.Tensor,
                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                slot_mapping: Optional[torch.Tensor]) -> None:
+                slot_mapping: Optional[torch.Tensor], pairs: bool = False) -> None:
     """In place on the fused down-projections [T, q_rank | kv_rank | rot_dim] (or [T, q_rank] for a
     layer that reads another layer's cache): the query latent is RMS-normed (weight ``qw``); the
     key/value latent is RMS-normed (weight ``kw``) and the shared key part behind it is rotated by
-    its position (``freq``: rotary_freq); both go to the pages at ``slot_mapping`` - the key page
+    its position (``freq``: rotary_freq; ``pairs``: entries 2i and 2i + 1 turn together instead of i
+    and i + len(freq)); both go to the pages at ``slot_mapping`` - the key page
     row is [latent | rotated part] (the page's rows may be wider: what lies behind is left as it is,
     zero), the value page holds the latent once more, dim-major."""
     T = proj.shape[0]
@@ -311,21 +423,21 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
             return
         c = proj[:, q_rank:q_rank + kv_rank].float()
         c = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kw.float()).to(proj.dtype)
-        kr = _rotate_half(proj[:, q_rank + kv_rank:].float(), positions, freq).to(proj.dtype)
+        kr = _rotate(proj[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim].float(), positions, freq, pairs).to(proj.dtype)
         proj[:, q_rank:q_rank + kv_rank] = c
-        proj[:, q_rank + kv_rank:] = kr
-        ok = slot_mapping >= 0
-        s = slot_mapping[ok].long()
+        proj[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim] = kr
+        ok = slot_mapping[:T] >= 0
+        s = slot_mapping[:T][ok].long()
         bs = k_cache.shape[1]
-        k_cache.view(-1, k_cache.shape[2])[s, :kv_rank + rot_dim] = proj[ok, q_rank:]
+        k_cache.view(-1, k_cache.shape[2])[s, :kv_rank + rot_dim] = proj[ok, q_rank:q_rank + kv_rank + rot_dim]
         v_cache.view(-1, kv_rank, bs)[s // bs, :, s % bs] = c[ok]
         return
     native().latent_prep(proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw, float(eps), positions, freq,
-                         k_cache, v_cache, slot_mapping)
+                         k_cache, v_cache, slot_mapping, bool(pairs))
 
 
 def latent_queries(q: torch.Tensor, q_lat: torch.Tensor, H: int, dim: int, rot_dim: int, positions: torch.Tensor,
-                   freq: torch.Tensor, pitch: int = 0) -> torch.Tensor:
+                   freq: torch.Tensor, pitch: int = 0, pairs: bool = False) -> torch.Tensor:
     """The queries against the latent cache: per head [q_lat | rotated part | zeros], [T, H * pitch]
     (``pitch`` 0: R + rot_dim, no padding; else the key pages' row width).
     ``q`` [T, H * (dim + rot_dim)] are the up-projected queries (their last ``rot_dim`` entries per
@@ -334,21 +446,32 @@ def latent_queries(q: torch.Tensor, q_lat: torch.Tensor, H: int, dim: int, rot_d
     T, R = q.shape[0], q_lat.shape[2]
     pitch = pitch or R + rot_dim
     if not q.is_cuda:
-        qr = _rotate_half(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, freq).to(q.dtype)
+        qr = _rotate(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, freq, pairs).to(q.dtype)
         pad = torch.zeros(T, H, pitch - R - rot_dim, dtype=q.dtype)
         return torch.cat([q_lat.transpose(0, 1), qr, pad], -1).reshape(T, H * pitch)
     out = torch.empty(T, H * pitch, dtype=q.dtype, device=q.device)
-    native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, freq)
+    native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, freq, bool(pairs))
     return out
+
+
+_NO_SINK: dict = {}
+
+
+def _no_sink(H: int, device) -> torch.Tensor:
+    key = (H, str(device))
+    if key not in _NO_SINK:
+        _NO_SINK[key] = torch.full((H,), -1.0e30, dtype=torch.float32, device=device)
+    return _NO_SINK[key]
 
 
 def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                      H: int, scale: float, window: int, sinks: Optional[torch.Tensor], cu: Optional[torch.Tensor] = None,
                      ctx: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None, fast: int = 1,
-                     split: int = 0) -> torch.Tensor:
+                     split: int = 0, sink: bool = True) -> torch.Tensor:
     """Attention of ``qa`` [T, H * pitch] (latent_queries) over the latent pages: every head reads
     the one key stream ``k_cache`` [blocks, bs, pitch] and the one value stream ``v_cache`` [blocks, 1,
-    kv_rank, bs]; sliding window and learned sinks as in window_attention_*.  ``cu`` / ``ctx``: prompt
+    kv_rank, bs]; sliding window and learned sinks as in window_attention_* (``sink`` False: an
+    ordinary softmax, nothing but the keys in the denominator).  ``cu`` / ``ctx``: prompt
     chunks (rows of segment s at positions ctx[s] ..); else ``seq_lens``: one row per sequence, at its
     newest token.  Returns [T, H * kv_rank].  GPU, bf16, pitch a multiple of 32 up to 320 and kv_rank a
     multiple of 16 up to 256 (``fast``): the matrix-core kernel, 16 heads of one token per tile
@@ -357,12 +480,17 @@ def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     large steps' chunks take 33, few rows 8); other sizes and fp32:
     the any-size kernels with one shared key/value head."""
     T, pitch, dv = qa.shape[0], k_cache.shape[2], v_cache.shape[2]
+    if not sink:
+        sinks = None
     if qa.is_cuda and fast and qa.dtype == torch.bfloat16:
         out = torch.empty(T, H * dv, dtype=qa.dtype, device=qa.device)
+        # the matrix-core kernels start every row from a sink term; without one that term gets a logit
+        # so low that its weight exp(logit - max) is exactly zero in fp32
+        sk = sinks if sink else _no_sink(H, qa.device)
         if native().latent_attention(out, qa, k_cache, v_cache, cu, ctx, seq_lens, block_tables, int(H), float(scale),
-                                     int(window), sinks, int(split)):
+                                     int(window), sk, int(split)):
             return out
-    args = (H, 1, pitch, dv, scale, window, True)
+    args = (H, 1, pitch, dv, scale, window, bool(sink))
     if cu is not None:
         return window_attention_prefill(qa, k_cache, v_cache, cu, ctx, block_tables, *args, mfma=fast, sinks=sinks)
     return window_attention_decode(qa, k_cache, v_cache, block_tables, seq_lens, *args, vec=bool(fast), sinks=sinks)
@@ -404,9 +532,10 @@ def conv_silu(proj: torch.Tensor, col0: int, C: int, conv_w: torch.Tensor, conv_
     return out
 
 
-def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
-             d_skip: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
-             seg_slot: torch.Tensor, nh: int, P: int, N: int, G: int, mode: int = 0) -> torch.Tensor:
+def ssm_scan(xbc: torch.Tensor, proj: Optional[torch.Tensor], dt_col: int, dt_bias: Optional[torch.Tensor],
+             a_log: Optional[torch.Tensor], d_skip: Optional[torch.Tensor], state: torch.Tensor, seg_cu: torch.Tensor,
+             seg_ctx: torch.Tensor, seg_slot: torch.Tensor, nh: int, P: int, N: int, G: int, mode: int = 0,
+             decay: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The selective state-space recurrence, fp32, token by token within each segment:
 
         dt = softplus(proj[t, dt_col + h] + dt_bias[h]);  S <- exp(-exp(a_log[h]) dt) S + dt B_t x_t^T
@@ -415,12 +544,18 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.
     ``xbc`` [T, nh*P | G*N | G*N] holds x, B, C (head h reads group h // (nh / G)); ``state``
     [slots, nh, N, P] fp32 is read at the segment's start (zero where seg_ctx is 0) and written
     back at its end.  Returns y [T, nh*P] fp32.  GPU: two lane mappings of the same arithmetic,
-    chosen by the step's mean segment length (``mode`` 1 / 2 forces the decode / the prompt one)."""
+    chosen by the step's mean segment length (``mode`` 1 / 2 forces the decode / the prompt one).
+
+    ``decay`` [nh] fp32 (then ``proj``, ``dt_bias``, ``a_log``, ``d_skip`` are not read): the
+    recurrence with a fixed decay per head, step size 1 and no skip term,
+    ``S <- decay[h] S + B_t x_t^T;  y_t = S^T C_t`` - linear attention with B, C, x = k, q, v
+    (linear_attention below)."""
     T = xbc.shape[0]
     if not xbc.is_cuda:
         y = torch.zeros(T, nh * P, dtype=torch.float32)
-        A = torch.exp(a_log.float())
-        Dk = d_skip.float()
+        fixed = decay is not None
+        A = torch.exp(a_log.float()) if not fixed else None
+        Dk = d_skip.float() if not fixed else torch.zeros(nh)
         cul = seg_cu.tolist()
         inner = nh * P
         for s, (c0, slot) in enumerate(zip(seg_ctx.tolist(), seg_slot.tolist())):
@@ -431,31 +566,52 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.
             xs = xbc[a:b, :inner].float().view(-1, nh, P)
             Bs = xbc[a:b, inner:inner + G * N].float().view(-1, G, N).repeat_interleave(nh // G, dim=1)
             Cs = xbc[a:b, inner + G * N:].float().view(-1, G, N).repeat_interleave(nh // G, dim=1)
-            dt = F.softplus(proj[a:b, dt_col:dt_col + nh].float() + dt_bias.float(), threshold=30.0)
-            dec = torch.exp(-A * dt)
+            if fixed:
+                dt = torch.ones(b - a, nh)
+                dec = decay.float().expand(b - a, nh)
+            else:
+                dt = F.softplus(proj[a:b, dt_col:dt_col + nh].float() + dt_bias.float(), threshold=30.0)
+                dec = torch.exp(-A * dt)
             for t in range(b - a):
                 S = dec[t, :, None, None] * S + dt[t, :, None, None] * Bs[t, :, :, None] * xs[t, :, None, :]
                 y[a + t] = (torch.einsum("hnp,hn->hp", S, Cs[t]) + Dk[:, None] * xs[t]).reshape(-1)
             state[slot] = S
         return y
     y = torch.empty(T, nh * P, dtype=torch.float32, device=xbc.device)
-    native().ssm_scan(y, xbc, proj, int(dt_col), dt_bias, a_log, d_skip, state, seg_cu, seg_ctx, seg_slot, nh, P, N, G,
-                      int(mode))
+    native().ssm_scan(y, xbc, proj, int(dt_col), dt_bias, a_log, d_skip, decay, state, seg_cu, seg_ctx, seg_slot, nh, P,
+                      N, G, int(mode))
     return y
 
 
+def linear_attention(vkq: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor,
+                     seg_ctx: torch.Tensor, seg_slot: torch.Tensor, H: int, dk: int, dv: int, mode: int = 0) -> torch.Tensor:
+    """Linear attention with a fixed decay per head, as a recurrence over each segment:
+
+        S_t = decay[h] S_(t-1) + k_t v_t^T;   o_t = S_t^T q_t
+
+    ``vkq`` [T, H*dv | H*dk | H*dk] holds v, k, q head by head (contiguous); ``state`` [slots, H, dk,
+    dv] fp32 is read at a segment's start (zero where seg_ctx is 0) and written back at its end.
+    Returns o [T, H*dv] fp32.  State, products and sums are fp32."""
+    return ssm_scan(vkq, None, 0, None, None, None, state, seg_cu, seg_ctx, seg_slot, H, dv, dk, H, mode, decay=decay)
+
+
 def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, w: torch.Tensor, eps: float, groups: int,
-                     out_dtype: torch.dtype) -> torch.Tensor:
+                     out_dtype: torch.dtype, after: bool = False) -> torch.Tensor:
     """``y`` [T, n] fp32 times silu of the gate ``proj[:, z_col : z_col + n]``, then RMS-normed in
-    ``groups`` equal parts (each by its own root mean square) times ``w`` [n]."""
+    ``groups`` equal parts (each by its own root mean square) times ``w`` [n].  ``after``: the norm
+    first (of ``y`` as it is), then times ``w`` and the SIGMOID of the gate."""
     T, n = y.shape
     if not y.is_cuda:
+        if after:
+            g = y.view(T, groups, n // groups)
+            g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+            return (g.reshape(T, n) * w.float() * torch.sigmoid(proj[:, z_col:z_col + n].float())).to(out_dtype)
         g = y * _silu(proj[:, z_col:z_col + n].float())
         g = g.view(T, groups, n // groups)
         g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
         return (g.reshape(T, n) * w.float()).to(out_dtype)
     out = torch.empty(T, n, dtype=out_dtype, device=y.device)
-    native().gated_group_norm(out, y, proj, int(z_col), w, float(eps), int(groups))
+    native().gated_group_norm(out, y, proj, int(z_col), w, float(eps), int(groups), bool(after))
     return out
 
 
