@@ -151,8 +151,9 @@ def _sub(tensors: dict, prefix: str) -> dict:
     return {k[len(prefix):]: v.to(F64) for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, tensors: dict, tokens: list) -> tuple:
-    """(logits [n, vocab], residual stream after every layer [layers, n, width]), float64."""
+def forward(cfg: dict, tensors: dict, tokens: list, return_layers: bool = False):
+    """Logits [n, vocab] in float64 (``return_layers``: and the residual stream after every layer,
+    [layers, n, width])."""
     eps, mult = float(cfg["norm"]["eps"]), float(cfg["residual_mult"])
     t = {k: v.to(F64) for k, v in tensors.items()}
     x = t["embed"][torch.tensor(tokens, dtype=torch.long)]
@@ -182,4 +183,63 @@ def forward(cfg: dict, tensors: dict, tokens: list) -> tuple:
     cap = float(cfg.get("logit_softcap") or 0.0)
     if cap > 0:
         z = cap * torch.tanh(z / cap)
-    return z, torch.stack(after)
+    return (z, torch.stack(after)) if return_layers else z
+
+
+def random_weights(cfg: dict, seed: int = 0) -> dict:
+    """Random tensors of a config's shapes (values a bf16 checkpoint could hold), by name."""
+    g = torch.Generator().manual_seed(seed)
+    d, V = cfg["width"], cfg["vocab"]
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(torch.bfloat16).float()
+
+    def one(mean=1.0):
+        return rnd(1, std=0.15, mean=mean).reshape(())
+
+    w = {"embed": rnd(V, d, std=0.8), "final.norm": one(), "head": rnd(V, d, std=2 * d ** -0.5)}
+    for i, spec in enumerate(cfg["layers"]):
+        L, m, P = f"l{i}.", spec["mixer"], f"l{i}.mix."
+        w[L + "norm1"] = one()
+        w[L + "rg1"], w[L + "rg1.b"] = rnd(d, d, std=d ** -0.5), rnd(d, std=0.7)
+        H = m["heads"]
+        if spec["type"] == "attention":
+            G, dk, dv = m["kv_heads"], m["dim"], m["vdim"]
+            w[P + "q"], w[P + "k"] = rnd(H * dk, d, std=1.5 * d ** -0.5), rnd(G * dk, d, std=1.5 * d ** -0.5)
+            w[P + "v"], w[P + "g"] = rnd(G * dv, d, std=d ** -0.5), rnd(H * dv, d, std=d ** -0.5)
+            w[P + "temp"] = rnd(H, std=0.4, mean=1.2)
+            w[P + "o"] = rnd(d, H * dv, std=(H * dv) ** -0.5)
+        elif spec["type"] == "lightning":
+            dk, dv = m["dim"], m["vdim"]
+            w[P + "q"], w[P + "k"] = rnd(H * dk, d, std=d ** -0.5), rnd(H * dk, d, std=d ** -0.5)
+            w[P + "v"], w[P + "g"] = rnd(H * dv, d, std=d ** -0.5), rnd(H * dv, d, std=d ** -0.5)
+            w[P + "norm"] = rnd(H * dv, std=0.1, mean=1.0)
+            w[P + "o"] = rnd(d, H * dv, std=(H * dv) ** -0.5)
+        else:
+            dn, dr, dv, R, Q = m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            w[P + "dq"], w[P + "dq.norm"] = rnd(Q, d, std=d ** -0.5), rnd(Q, std=0.1, mean=1.0)
+            w[P + "uq"] = rnd(H * (dn + dr), Q, std=1.5 * Q ** -0.5)
+            if m.get("kv_from") is None:
+                w[P + "dkv"], w[P + "dkv.norm"] = rnd(R + dr, d, std=d ** -0.5), rnd(R, std=0.1, mean=1.0)
+            w[P + "uk"] = rnd(H * dn, R, std=1.5 * R ** -0.5)
+            w[P + "uv"] = rnd(H * dv, R, std=R ** -0.5)
+            w[P + "o"] = rnd(d, H * dv, std=(H * dv) ** -0.5)
+        ml = spec.get("mlp")
+        if ml is None:
+            continue
+        f = ml["ff"]
+        w[L + "norm2"] = one()
+        w[L + "rg2"], w[L + "rg2.b"] = rnd(d, d, std=d ** -0.5), rnd(d, std=0.7)
+        w[L + "mlp.gate"], w[L + "mlp.up"] = rnd(f, d, std=1.5 * d ** -0.5), rnd(f, d, std=d ** -0.5)
+        w[L + "mlp.down"] = rnd(d, f, std=f ** -0.5)
+    return w
+
+
+def greedy(cfg: dict, w: dict, prompt, n: int) -> list:
+    """``n`` tokens by repeated whole-sequence forwards, each the argmax of the last logits."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = int(torch.argmax(forward(cfg, w, seq)[-1]))
+        out.append(t)
+        seq.append(t)
+    return out
