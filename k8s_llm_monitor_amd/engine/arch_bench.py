@@ -2,7 +2,10 @@
 layer sizes, random weights, one GPU (``python bench.py --mode arch [--arch-design NAME]``):
 Dunesun beside a Mixtral-style model (attention + routed experts in every layer); Kisutar beside
 an all-attention Dunesun model (windowed attention with sinks, fp32 residual stream, routed experts
-with a shared expert in every layer - the same kernels family).  Both models run through the same
+with a shared expert in every layer - the same kernels family); Bitonex (rotary attention, linear
+attention and latent attention layers in turn, dense gated feed-forward) beside a Dunesun model of
+attention and Mamba-2 layers with the same heads, head sizes, recurrent state size and feed-forward
+width (one expert, so every token takes it).  Both models run through the same
 ModelRunner step functions the engine uses: one prefill step of ``seqs`` whole prompts, then decode
 steps of ``batch`` sequences (hipGraph replay where the model's decode is captured)."""
 from __future__ import annotations
@@ -73,6 +76,53 @@ def _kisutar_pair(size: str, window: int) -> tuple:
     return new, ref
 
 
+# Bitonex: (name, width, heads, kv heads, head dim, rotating dims, latent unrotated dim, rotated dim, q rank, kv rank,
+#           ff, layers); layers take attention, linear attention, latent attention in turn
+BITONEX_SIZES = {
+    "s": ("d1024", 1024, 8, 2, 128, 64, 96, 32, 384, 128, 2816, 6),
+    "m": ("d2048", 2048, 16, 4, 128, 64, 96, 32, 768, 256, 5632, 6),
+    "l": ("d4096", 4096, 32, 8, 128, 64, 96, 32, 1536, 256, 11008, 3),
+}
+
+
+def _bitonex_pair(size: str, window: int) -> tuple:
+    """Bitonex (the second latent layer reads the first one's pages) and a Dunesun model whose layers
+    are attention, Mamba-2 (as many state entries per token as the linear attention layer), attention,
+    each with ONE expert of the dense layers' width."""
+    name, d, H, G, D, rd, dn, dr, Q, R, ff, L = BITONEX_SIZES[size]
+    pair = lambda m: tuple(sorted(m.items()))
+    decay = tuple(1.0 - 2.0 ** (-3 - 5 * h / max(1, H - 1)) for h in range(H))
+    first_latent = 2
+
+    def layer(i):
+        if i % 3 == 0:
+            return LayerSpec("attention", pair({"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                                                "rot.dims": rd, "rot.base": 1e6}), DenseSpec(ff))
+        if i % 3 == 1:
+            return LayerSpec("lightning", pair({"heads": H, "dim": D, "vdim": D, "decay": decay}), DenseSpec(ff))
+        m = {"heads": H, "dim": dn, "rot_dim": dr, "vdim": D, "q_rank": Q, "kv_rank": R, "scale": (dn + dr) ** -0.5,
+             "rot.base": 1e4, "rot.dims": dr}
+        if i > first_latent:
+            m["kv_from"] = first_latent
+        return LayerSpec("latent_attention", pair(m), DenseSpec(ff))
+
+    new = HybridConfig(name=f"bitonex-{name}", arch="bitonex", vocab_size=32000, d_model=d,
+                       layers=tuple(layer(i) for i in range(L)), max_position=8192, norm_eps=1e-6, residual_mult=0.5,
+                       logit_softcap=30.0)
+    one = MoESpec(1, 1, ff, 0)
+    # Bitonex attends to the whole prefix: so does the reference (no window, whatever ``window`` says)
+    att = LayerSpec("attention", pair({"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask.size": 0,
+                                       "scale": D ** -0.5}), one)
+    ssm = LayerSpec("mamba2", pair({"heads": H * D // 64, "vdim": 64, "state": D, "groups": 1, "conv": 4,
+                                    "norm_groups": 1}), one)
+    ref = HybridConfig(name=f"dunesun-hybrid-{name}", arch="dunesun", vocab_size=32000, d_model=d,
+                       layers=tuple(ssm if i % 3 == 1 else att for i in range(L)), max_position=8192)
+    return new, ref
+
+
+PAIRS = {"dunesun": _pair, "kisutar": _kisutar_pair, "bitonex": _bitonex_pair}
+
+
 def _measure(cfg, seqs: int, prompt: int, batch: int, steps: int, warmup: int, graphs: bool) -> dict:
     dev = torch.device("cuda:0")
     model = build_model(cfg, device=dev, dtype=torch.bfloat16)
@@ -141,7 +191,7 @@ def run(a) -> None:
     """``a``: bench.py's parsed arguments (arch_sizes, arch_prompt, arch_seqs, batch, steps, warmup)."""
     rows = []
     for size in a.arch_sizes.split(","):
-        hy, ref = (_kisutar_pair if getattr(a, "arch_design", "dunesun") == "kisutar" else _pair)(size, a.arch_window)
+        hy, ref = PAIRS[getattr(a, "arch_design", "dunesun")](size, a.arch_window)
         for cfg in ((hy, ref) if a.arch_which == "both" else ((hy,) if a.arch_which == "new" else (ref,))):
             r = _measure(cfg, a.arch_seqs, a.arch_prompt, a.batch, a.steps, a.warmup, not a.no_graphs)
             r["size"] = size
