@@ -42,6 +42,8 @@ int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_strid
                        const float* a_log, const float* d_skip, const float* decay, float* state, const int* cu,
                        const int* ctx, const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode,
                        hipStream_t s);
+int k8sllm_hy_linear_attn_chunk(float* y, const void* vkq, const float* decay, float* state, const int* cu,
+                                const int* ctx, const int* slot, int S, int H, int dk, int dv, int nt, hipStream_t s);
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
                      const float* bias, int E, int K, int rows_w, int over_all, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
@@ -406,6 +408,28 @@ void ssm_scan(Tensor y, Tensor xbc, OptT proj, int64_t dt_col, OptT dt_bias, Opt
         "ssm_scan");
 }
 
+// The matrix-core (chunked) linear attention for bf16 prompts; false: these sizes or dtype are not the
+// kernel's, nothing was launched.
+bool linear_attention_chunked(Tensor y, Tensor vkq, Tensor decay, Tensor state, Tensor cu, Tensor ctx, Tensor slot,
+                              int64_t H, int64_t dk, int64_t dv, int64_t nt) {
+  if (act(vkq, "vkq") != 0) return false;
+  f32c(y, "y");
+  f32c(decay, "decay");
+  f32c(state, "state");
+  segs(cu, ctx, slot);
+  const int64_t T = vkq.size(0);
+  TORCH_CHECK(vkq.dim() == 2 && vkq.is_contiguous() && vkq.size(1) == H * dv + 2 * H * dk, "vkq [T, H*dv + 2*H*dk]");
+  TORCH_CHECK(y.numel() == T * H * dv && decay.numel() == H, "linear attention: y [T, H*dv], decay [H]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv,
+              "state [slots, H, dk, dv]");
+  const int rc = k8sllm_hy_linear_attn_chunk(y.data_ptr<float>(), vkq.data_ptr(), decay.data_ptr<float>(),
+                                             state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(),
+                                             slot.data_ptr<int>(), (int)ctx.numel(), (int)H, (int)dk, (int)dv, (int)nt, cur());
+  if (rc == 1) return false;
+  check(rc, "linear_attention_chunked");
+  return true;
+}
+
 // In place on the fused rows [T, Hq*dk | G*dk | G*dv | ...]: rotary positions on the first 2 * len(freq)
 // entries of every q / k head (pairs: entry 2i with 2i + 1, else i with i + len(freq)), q heads times
 // q_scale [Hq] (optional), k and v to the pages.
@@ -676,6 +700,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sigmoid_gate", &sigmoid_gate);
   m.def("softcap", &softcap);
   m.def("rotary_cache", &rotary_cache);
+  m.def("linear_attention_chunked", &linear_attention_chunked);
   m.def("qk_norm_cache", &qk_norm_cache);
   m.def("window_attention_prefill", &window_attention_prefill);
   m.def("window_attention_decode", &window_attention_decode);

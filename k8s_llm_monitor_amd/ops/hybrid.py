@@ -584,15 +584,28 @@ def ssm_scan(xbc: torch.Tensor, proj: Optional[torch.Tensor], dt_col: int, dt_bi
 
 
 def linear_attention(vkq: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor,
-                     seg_ctx: torch.Tensor, seg_slot: torch.Tensor, H: int, dk: int, dv: int, mode: int = 0) -> torch.Tensor:
+                     seg_ctx: torch.Tensor, seg_slot: torch.Tensor, H: int, dk: int, dv: int, mode: int = 0,
+                     col_tiles: int = 0) -> torch.Tensor:
     """Linear attention with a fixed decay per head, as a recurrence over each segment:
 
         S_t = decay[h] S_(t-1) + k_t v_t^T;   o_t = S_t^T q_t
 
     ``vkq`` [T, H*dv | H*dk | H*dk] holds v, k, q head by head (contiguous); ``state`` [slots, H, dk,
     dv] fp32 is read at a segment's start (zero where seg_ctx is 0) and written back at its end.
-    Returns o [T, H*dv] fp32.  State, products and sums are fp32."""
-    return ssm_scan(vkq, None, 0, None, None, None, state, seg_cu, seg_ctx, seg_slot, H, dv, dk, H, mode, decay=decay)
+    Returns o [T, H*dv] fp32.  State, products and sums are fp32.
+
+    GPU: the sequential scan (``ssm_scan`` with the decay table; ``mode`` 1 / 2 force its decode /
+    prompt lane mapping), or - bf16 prompts (a mean of 32 rows per segment and more), ``dim`` a multiple
+    of 32 up to 128, ``vdim`` a multiple of 16; ``mode`` 3 forces it, ``col_tiles`` 1 / 2 its value
+    columns per workgroup (16 / 32; 0: 16) - chunks of 64 tokens on the matrix
+    cores: q.k on the bf16 instruction, everything that holds scores or state on the fp32 one, only the
+    state crossing chunks (the order of the fp32 sums then follows the chunk grid, which starts at the
+    segment's first row)."""
+    if vkq.is_cuda and vkq.dtype == torch.bfloat16 and (mode == 3 or (mode == 0 and vkq.shape[0] >= 32 * seg_ctx.numel())):
+        y = torch.empty(vkq.shape[0], H * dv, dtype=torch.float32, device=vkq.device)
+        if native().linear_attention_chunked(y, vkq, decay, state, seg_cu, seg_ctx, seg_slot, H, dk, dv, int(col_tiles)):
+            return y
+    return ssm_scan(vkq, None, 0, None, None, None, state, seg_cu, seg_ctx, seg_slot, H, dv, dk, H, mode if mode < 3 else 0, decay=decay)
 
 
 def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, w: torch.Tensor, eps: float, groups: int,

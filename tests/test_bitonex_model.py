@@ -589,6 +589,35 @@ def test_gpu_new_ops_match_their_torch_forms(dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,dk,dv,tiles", [(2, 32, 32, 0), (3, 64, 96, 2), (1, 96, 32, 1), (2, 128, 128, 1), (4, 128, 64, 2),
+                                           (3, 96, 48, 0), (2, 32, 16, 1)])
+def test_gpu_chunked_linear_attention_matches_the_recurrence(H, dk, dv, tiles):
+    """The matrix-core form (chunks of 64 tokens) against the token-by-token torch form: segments
+    shorter than, equal to and longer than a chunk, one continuing from its slot, one padding
+    segment, decays of 0, 1 and between; outputs and the states left in the slots."""
+    g = torch.Generator().manual_seed(5)
+    lens = [1, 63, 64, 65, 200, 7, 130]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    ctx = torch.tensor([0, 5, 0, 64, 0, 3, 9], dtype=torch.int32)
+    slot = torch.tensor([0, 1, 2, 3, 4, -1, 5], dtype=torch.int32)
+    T = int(cu[-1])
+    vkq = (torch.randn(T, H * dv + 2 * H * dk, generator=g) * 0.7).to(torch.bfloat16)
+    decay = torch.tensor(([0.9, 1.0, 0.0, 0.999] * 2)[:H])
+    st = torch.randn(6, H, dk, dv, generator=g)
+    want_state = st.clone()
+    want = hops.linear_attention(vkq, decay, want_state, cu, ctx, slot, H, dk, dv)
+    got_state = st.to("cuda")
+    got = hops.linear_attention(vkq.to("cuda"), decay.to("cuda"), got_state, cu.to("cuda"), ctx.to("cuda"), slot.to("cuda"),
+                                H, dk, dv, mode=3, col_tiles=tiles)
+    close(got.cpu(), want.double(), tol=2e-5)
+    close(got_state.cpu(), want_state.double(), tol=2e-5)
+    scan_state = st.to("cuda")
+    scan = hops.linear_attention(vkq.to("cuda"), decay.to("cuda"), scan_state, cu.to("cuda"), ctx.to("cuda"), slot.to("cuda"),
+                                 H, dk, dv, mode=2)
+    close(got.cpu(), scan.cpu().double(), tol=2e-5)
+
+
+@pytest.mark.gpu
 def test_gpu_greedy_generation_with_graphs():
     eng = LLMEngine(EngineConfig(model="bitonex-tiny", max_num_seqs=4, max_model_len=256, num_blocks=64,
                                  dtype="float32", max_prefill_tokens=32, mixed_prefill_tokens=16), device="cuda")
