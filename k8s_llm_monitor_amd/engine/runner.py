@@ -271,6 +271,7 @@ class ModelRunner:
         dv = {k: d[off[k]:off[k] + n] for k, n in sizes.items()}
         meta = AttnMeta(is_prefill=True, positions=dv["pos"], slot_mapping=dv["slots"], cu_seqlens=dv["cu"],
                         qb_seq=dv["qs"], qb_start=dv["st"], logits_idx=dv["lidx"].long())
+        meta.all_fresh = not any(starts)
         if paged:
             meta.ctx_start = dv["cst"]
             meta.block_tables = dv["bt"].view(len(seqs), W)

@@ -184,6 +184,26 @@ class Mamba2Mixer:
         return F.linear(g, self.wo)
 
 
+def _fresh_pages(meta: AttnMeta, T: int, device) -> tuple:
+    """Temporary pages for a step of whole prompts: (slot of every row, block tables [S, W], blocks),
+    every segment starting on a page of its own.  Computed once per step (cached on ``meta``), on the
+    device, from the segment offsets."""
+    got = getattr(meta, "_fresh_pages", None)
+    if got is None:
+        cu = meta.cu_seqlens.long()
+        S = cu.numel() - 1
+        nblk = (cu[1:] - cu[:-1] + BLOCK - 1) // BLOCK
+        first = torch.cumsum(nblk, 0) - nblk  # a segment's first temporary block
+        rows = torch.arange(T, device=device)
+        seg = torch.bucketize(rows, cu[1:], right=True).clamp(max=S - 1)
+        slots = (first[seg] * BLOCK + rows - cu[:-1][seg]).to(torch.int32)
+        nb = T // BLOCK + S
+        W = meta.block_tables.shape[1]
+        bt = (first[:, None] + torch.arange(W, device=device)[None, :]).clamp(max=nb - 1).to(torch.int32)
+        got = meta._fresh_pages = (slots, bt.contiguous(), nb)
+    return got
+
+
 class LatentAttention:
     """Attention over a compressed key/value stream (one normed latent of ``kv_rank`` and one
     rotated key part of ``rot_dim`` per token, shared by all heads), rotary positions on the
@@ -192,9 +212,17 @@ class LatentAttention:
     rotation layout (``rotary`` "half" / "pairs") and ``sink``.
     ``kv_from``: j - no key/value projection of its own; reads layer j's pages.
     ``tail``: extra rows [n, d] for the down-projection; forward leaves their outputs in ``tail_out``
-    (a [T, n] view) - the block's residual gate rides in the mixer's first GEMM."""
+    (a [T, n] view) - the block's residual gate rides in the mixer's first GEMM.
+
+    Two forms of the same attention.  Over the cache the per-head expansions are moved to the query
+    side (module docstring): every step can take it.  A step of whole prompts (every chunk starts at
+    position 0, no decode rows beside them; bf16, head sizes of the matrix-core kernel) of at least
+    ``EXPAND_MIN_ROWS`` rows instead expands this step's keys ``[W_uk c | shared part]`` and values
+    ``W_uv c`` per head into temporary pages and runs windowed attention's kernel over them:
+    ``dim + rot_dim + vdim`` multiply-adds per (query, key, head) instead of ``2 kv_rank + rot_dim``."""
 
     kind = "latent_attention"
+    EXPAND_MIN_ROWS = 1024
 
     def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
                  tail: Optional[torch.Tensor] = None):
@@ -256,6 +284,8 @@ class LatentAttention:
         hops.latent_prep(down, Q, R, dr, self.qn, self.kn, self.eps, meta.positions, self.freq,
                          kc if own else None, vc if own else None, meta.slot_mapping if own else None, pairs=self.pairs)
         q = F.linear(down[:, :Q], self.w_uq)
+        if self._expand_ok(h, meta):
+            return self._forward_expanded(q, down, meta, kc)
         # the per-head key expansion moved to the query: q_lat[h] = q_unrotated[h] @ W_uk[h]  ([H, T, R])
         q_lat = torch.bmm(q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1), self.w_uk.view(H, dn, R))
         qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq, self.pitch, pairs=self.pairs)
@@ -274,6 +304,36 @@ class LatentAttention:
         v = torch.empty(T, H, dv, dtype=h.dtype, device=h.device)
         torch.bmm(o.view(T, H, R).transpose(0, 1), self.w_uv.view(H, dv, R).transpose(1, 2), out=v.transpose(0, 1))
         return F.linear(v.view(T, H * dv), self.wo)
+
+    def _expand_ok(self, h: torch.Tensor, meta: AttnMeta) -> bool:
+        return (meta.is_prefill and meta.all_fresh and not meta.num_decode and h.is_cuda and h.dtype == torch.bfloat16
+                and bool(self.fast) and h.shape[0] >= self.EXPAND_MIN_ROWS
+                and (self.dn + self.dr) in (64, 128) and self.dv in (64, 128))
+
+    def _forward_expanded(self, q: torch.Tensor, down: torch.Tensor, meta: AttnMeta, kc: torch.Tensor) -> torch.Tensor:
+        """Whole prompts: per-head keys and values of this step's rows in temporary pages, windowed
+        attention's matrix-core kernel over them.  ``q`` [T, H * (dim + rot_dim)] still unturned."""
+        H, dn, dr, dv, Q, R = self.H, self.dn, self.dr, self.dv, self.Q, self.R
+        T, D = q.shape[0], self.dn + self.dr
+        if self.kv_from is None:  # latent_prep left the normed latent and the turned shared part in place
+            c, kr = down[:, Q:Q + R], down[:, Q + R:Q + R + dr]
+        else:  # the other layer's, as its pages hold them
+            rows = kc.view(-1, kc.shape[2]).index_select(0, meta.slot_mapping[:T].long())
+            c, kr = rows[:, :R], rows[:, R:R + dr]
+        fused = torch.empty(T, 2 * H * D + H * dv, dtype=q.dtype, device=q.device)  # [q | k | v], head by head
+        fused[:, :H * D] = q
+        kx = fused[:, H * D:2 * H * D].view(T, H, D)
+        kx[:, :, :dn] = F.linear(c, self.w_uk).view(T, H, dn)
+        kx[:, :, dn:] = kr.unsqueeze(1)
+        fused[:, 2 * H * D:] = F.linear(c, self.w_uv)
+        slots, bt, nb = _fresh_pages(meta, T, q.device)
+        kt = torch.zeros(nb, BLOCK, H * D, dtype=q.dtype, device=q.device)
+        vt = torch.zeros(nb, H, dv, BLOCK, dtype=q.dtype, device=q.device)
+        # the queries' rotated parts turn here; the shared key part was turned by latent_prep
+        hops.rotary_cache(fused, H, H, D, dv, meta.positions, self.freq, self.pairs, None, kt, vt, slots, rot_off=dn, rot_k=False)
+        o = hops.window_attention_prefill(fused, kt, vt, meta.cu_seqlens, meta.ctx_start, bt, H, H, D, dv, self.scale,
+                                          self.window, self.sink, mfma=self.fast, sinks=self.sinks)
+        return F.linear(o, self.wo)
 
 
 class RotaryAttention:

@@ -80,6 +80,8 @@ class AttnMeta:
     seg_cu: Optional[torch.Tensor] = None
     seg_ctx: Optional[torch.Tensor] = None
     seg_slot: Optional[torch.Tensor] = None
+    # prefill: every chunk of this step starts at position 0 (whole prompts, nothing cached before)
+    all_fresh: bool = False
 
 
 def _seed_for(name: str, seed: int) -> int:

@@ -22,8 +22,8 @@ int k8sllm_hy_activation_cols(void* out, const void* x, long x_stride, long rows
 int k8sllm_hy_sigmoid_gate(void* x, const void* z, long z_stride, long rows, int n, int vec, int f32, hipStream_t s);
 int k8sllm_hy_softcap(float* x, long n, float cap, hipStream_t s);
 int k8sllm_hy_rotary_cache(void* qkv, long stride, long T, int Hq, int G, int dk, int dv, const int* positions,
-                           const float* freq, int nf, int pairs, const float* q_scale, void* k_cache, void* v_cache,
-                           const int* slots, int bs, int f32, hipStream_t s);
+                           const float* freq, int nf, int pairs, int rot_off, int rot_k, const float* q_scale,
+                           void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_swiglu(void* out, const void* gu, long rows, int f, int f32, hipStream_t s);
 int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float* kw, float eps, long T, int nq,
                             int nk, int nv, void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
@@ -432,15 +432,17 @@ bool linear_attention_chunked(Tensor y, Tensor vkq, Tensor decay, Tensor state, 
 
 // In place on the fused rows [T, Hq*dk | G*dk | G*dv | ...]: rotary positions on the first 2 * len(freq)
 // entries of every q / k head (pairs: entry 2i with 2i + 1, else i with i + len(freq)), q heads times
-// q_scale [Hq] (optional), k and v to the pages.
+// q_scale [Hq] (optional), k and v to the pages.  rot_off: the turning entries start there in every head;
+// rot_k false: the keys are copied as they are.
 void rotary_cache(Tensor qkv, int64_t Hq, int64_t G, int64_t dk, int64_t dv, Tensor positions, Tensor freq, bool pairs,
-                  OptT q_scale, OptT k_cache, OptT v_cache, OptT slots) {
+                  OptT q_scale, OptT k_cache, OptT v_cache, OptT slots, int64_t rot_off, bool rot_k) {
   const int f = act(qkv, "qkv");
   f32c(freq, "freq");
   i32c(positions, "positions");
   const int64_t nq = Hq * dk, nk = G * dk, nv = G * dv, T = qkv.size(0);
   TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= nq + nk + nv, "qkv [T, Hq*dk + G*dk + G*dv (+ more)]");
-  TORCH_CHECK(Hq >= 1 && G >= 1 && positions.numel() >= T && 2 * freq.numel() <= dk, "rotary_cache: heads / positions / freq");
+  TORCH_CHECK(Hq >= 1 && G >= 1 && positions.numel() >= T && rot_off >= 0 && rot_off + 2 * freq.numel() <= dk,
+              "rotary_cache: heads / positions / freq");
   const float* qs = nullptr;
   if (q_scale.has_value()) {
     f32c(*q_scale, "q_scale");
@@ -459,7 +461,7 @@ void rotary_cache(Tensor qkv, int64_t Hq, int64_t G, int64_t dk, int64_t dv, Ten
     vc = v_cache->data_ptr();
   }
   check(k8sllm_hy_rotary_cache(qkv.data_ptr(), qkv.stride(0), T, (int)Hq, (int)G, (int)dk, (int)dv, positions.data_ptr<int>(),
-                               freq.data_ptr<float>(), (int)freq.numel(), pairs, qs, kc, vc, sp,
+                               freq.data_ptr<float>(), (int)freq.numel(), pairs, (int)rot_off, rot_k, qs, kc, vc, sp,
                                k_cache.has_value() ? (int)k_cache->size(1) : 16, f, cur()),
         "rotary_cache");
 }

@@ -268,20 +268,30 @@ def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: fl
 
 def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positions: torch.Tensor, freq: torch.Tensor,
                  pairs: bool, q_scale: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
-                 v_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> None:
+                 v_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], rot_off: int = 0,
+                 rot_k: bool = True) -> None:
     """In place on the fused rows [T, Hq*dk | Hkv*dk | Hkv*dv | ...]: the first ``2 len(freq)`` entries
     of every query and key head turn by the angle ``position * freq[i]`` (fp32; ``pairs``: entry 2i
     with 2i + 1, else entry i with i + len(freq); rotary_freq); the rest of a head passes.  ``q_scale``
     [Hq] fp32 (optional): every query head is multiplied by its number in the same pass (a per-head
     temperature folded into the query).  Keys (turned) and values go to the paged cache at
-    ``slot_mapping`` (< 0: not written)."""
+    ``slot_mapping`` (< 0: not written).  ``rot_off``: the turning entries are ``rot_off .. rot_off +
+    2 len(freq)`` of every head instead of the first; ``rot_k`` False: the keys are taken as they are
+    (turned already) and only written to the pages."""
     nq, nk, nv = Hq * dk, Hkv * dk, Hkv * dv
     if not qkv.is_cuda:
         T = qkv.shape[0]
-        q = _rotate(qkv[:, :nq].float().view(T, Hq, dk), positions, freq, pairs)
+
+        def turn(x):
+            x = x.clone()
+            x[..., rot_off:] = _rotate(x[..., rot_off:], positions, freq, pairs)
+            return x
+
+        q = turn(qkv[:, :nq].float().view(T, Hq, dk))
         if q_scale is not None:
             q = q * q_scale.float().view(1, Hq, 1)
-        k = _rotate(qkv[:, nq:nq + nk].float().view(T, Hkv, dk), positions, freq, pairs)
+        k = qkv[:, nq:nq + nk].float().view(T, Hkv, dk)
+        k = turn(k) if rot_k else k
         qkv[:, :nq] = q.reshape(T, nq).to(qkv.dtype)
         qkv[:, nq:nq + nk] = k.reshape(T, nk).to(qkv.dtype)
         if k_cache is not None:
@@ -291,7 +301,8 @@ def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positio
             bs = k_cache.shape[1]
             v_cache.view(-1, nv, bs)[s // bs, :, s % bs] = qkv[ok, nq + nk:nq + nk + nv]
         return
-    native().rotary_cache(qkv, Hq, Hkv, dk, dv, positions, freq, bool(pairs), q_scale, k_cache, v_cache, slot_mapping)
+    native().rotary_cache(qkv, Hq, Hkv, dk, dv, positions, freq, bool(pairs), q_scale, k_cache, v_cache, slot_mapping,
+                          int(rot_off), bool(rot_k))
 
 
 def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sink: bool,

@@ -90,6 +90,54 @@ def test_odd_sizes_everywhere():
         close(rig.run_cut("a", t, cuts), want)
 
 
+def test_models_without_pages_or_without_state():
+    """Only recurrent layers (no layer owns pages), and no recurrent layer (no state slots)."""
+    for layers in ([lin(mlp=dense(9)), lin(2, 4, 6, (0.6, 0.8))], [lat(mlp=dense(9)), att(), lat(2, 8, 8, 6, 12, 24, 0.3, kv_from=0)]):
+        cfg = make_cfg(layers)
+        rig = rig_for(cfg, 4)
+        assert (rig.runner.num_state_slots > 0) == (layers[0]["type"] == "lightning")
+        t, u = toks(37, cfg["vocab"], 2), toks(20, cfg["vocab"], 3)
+        want, wu = O.forward(cfg, rig.w, t), O.forward(cfg, rig.w, u)
+        close(rig.run_cut("a", t, [18, 2]), want)
+        a = rig.step([("a", t[:30]), ("b", u[:5])])
+        b = rig.step([("a", t[30:31]), ("b", u[5:])], end=["b"])
+        c = rig.step([("a", t[31:])], end=["a"])
+        close(torch.cat([a["a"], b["a"], c["a"]]), want)
+        close(torch.cat([a["b"], b["b"]]), wu)
+
+
+def _force_expanded(monkeypatch):
+    """Latent attention takes its expanded form (per-head keys and values in temporary pages) for
+    every step of whole prompts, whatever the sizes and the dtype."""
+    from k8s_llm_monitor_amd.models.hybrid import LatentAttention
+
+    calls = []
+    real = LatentAttention._forward_expanded
+    monkeypatch.setattr(LatentAttention, "_forward_expanded", lambda self, *a: calls.append(1) or real(self, *a))
+    monkeypatch.setattr(LatentAttention, "_expand_ok",
+                        lambda self, h, meta: meta.is_prefill and meta.all_fresh and not meta.num_decode)
+    return calls
+
+
+def test_latent_expanded_form_equals_the_oracle(monkeypatch):
+    """The expanded form in 32-bit, any sizes: unequal whole prompts in one step (every segment on
+    temporary pages of its own), a layer reading another layer's latent, then portions and decoding
+    over the latent cache those steps left."""
+    calls = _force_expanded(monkeypatch)
+    cfg = make_cfg([lat(3, 5, 6, 3, 9, 7, 0.4, mlp=dense(13)), att(), lat(5, 3, 6, 7, 5, 7, 0.3, kv_from=0), lat(mlp=dense(8))])
+    rig = rig_for(cfg, 12)
+    t, u, v = toks(50, cfg["vocab"], 4), toks(17, cfg["vocab"], 5), toks(33, cfg["vocab"], 6)
+    want = {n: O.forward(cfg, rig.w, x) for n, x in (("a", t), ("b", u), ("c", v))}
+    a = rig.step([("a", t[:40]), ("b", u[:16]), ("c", v[:33])], end=["c"])
+    assert len(calls) == 3
+    b = rig.step([("a", t[40:41]), ("b", u[16:])], end=["b"])
+    c = rig.step([("a", t[41:])], end=["a"])
+    assert len(calls) == 3
+    close(torch.cat([a["a"], b["a"], c["a"]]), want["a"])
+    close(torch.cat([a["b"], b["b"]]), want["b"])
+    close(a["c"], want["c"])
+
+
 def test_layer_outputs_match_oracle():
     rig = rig_for(FULL, 5)
     t = toks(19, FULL["vocab"], 3)
@@ -506,6 +554,57 @@ def test_gpu_matrix_core_sizes_bf16():
         close_most(rig.run_cut("a", t, cuts), want, 0.05, frac=1.0)
     r32 = rig_for(cfg, 6, device="cuda", dtype=torch.float32, num_blocks=48)
     close(r32.run_cut("a", t, [70, 3]), want)
+
+
+@pytest.mark.gpu
+def test_gpu_latent_whole_prompts_take_the_expanded_form(monkeypatch):
+    """A step of whole prompts runs latent attention with per-head keys and values in temporary pages
+    (unequal prompts in one step: every segment on pages of its own; a layer reading another layer's
+    latent); portions and decoding go over the latent cache.  Both forms against the oracle and
+    against each other."""
+    from k8s_llm_monitor_amd.models.hybrid import LatentAttention
+
+    cfg = make_cfg([lat(4, 32, 32, 64, 48, 64, 0.12, 1e4, mlp=dense(64)), att(4, 2, 64, 64, 32, 1e4, 0.125),
+                    lat(2, 96, 32, 128, 40, 64, 0.09, 1e4, kv_from=0, mlp=dense(48))], width=128, vocab=211, mult=0.35)
+    w = O.random_weights(cfg, 9)
+    t, u = toks(150, cfg["vocab"], 4), toks(70, cfg["vocab"], 5)
+    want, wu = O.forward(cfg, w, t), O.forward(cfg, w, u)
+    calls = []
+    real = LatentAttention._forward_expanded
+    monkeypatch.setattr(LatentAttention, "_forward_expanded", lambda self, *a: calls.append(1) or real(self, *a))
+
+    def run(min_rows):
+        monkeypatch.setattr(LatentAttention, "EXPAND_MIN_ROWS", min_rows)
+        rig = rig_for(cfg, w=w, device="cuda", dtype=torch.bfloat16, num_blocks=48)
+        a = rig.step([("a", t[:140]), ("b", u[:64])])  # whole prompts, unequal, one step
+        b = rig.step([("a", t[140:141]), ("b", u[64:])], end=["b"])  # a decode row beside a portion
+        c = rig.step([("a", t[141:])], end=["a"])
+        return torch.cat([a["a"], b["a"], c["a"]]), torch.cat([a["b"], b["b"]])
+
+    ga, gb = run(32)
+    assert len(calls) == 2  # both latent layers, the first step only
+    ha, hb = run(1 << 30)
+    assert len(calls) == 2
+    for got, ref in ((ga, want), (gb, wu), (ha, want), (hb, wu)):
+        close_most(got, ref, 0.05, frac=1.0)
+    close_most(ga, ha.double(), 0.02, frac=1.0)
+    close_most(gb, hb.double(), 0.02, frac=1.0)
+
+
+@pytest.mark.gpu
+def test_gpu_latent_expanded_form_fp32(monkeypatch):
+    calls = _force_expanded(monkeypatch)
+    cfg = make_cfg([lat(3, 5, 6, 3, 9, 7, 0.4, mlp=dense(13)), att(), lat(5, 3, 6, 7, 5, 7, 0.3, kv_from=0),
+                    lat(2, 32, 32, 64, 24, 32, 0.2)])
+    rig = rig_for(cfg, 12, device="cuda", dtype=torch.float32)
+    t, u = toks(50, cfg["vocab"], 4), toks(17, cfg["vocab"], 5)
+    wt, wu = O.forward(cfg, rig.w, t), O.forward(cfg, rig.w, u)
+    a = rig.step([("a", t[:40]), ("b", u[:16])])
+    b = rig.step([("a", t[40:41]), ("b", u[16:])], end=["b"])
+    c = rig.step([("a", t[41:])], end=["a"])
+    assert len(calls) == 3
+    close(torch.cat([a["a"], b["a"], c["a"]]), wt)
+    close(torch.cat([a["b"], b["b"]]), wu)
 
 
 @pytest.mark.gpu

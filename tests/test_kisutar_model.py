@@ -182,6 +182,30 @@ def test_prefill_equals_token_by_token_and_portions():
         close(rig.run_cut("a", t, cuts), want)
 
 
+def test_whole_prompts_in_the_expanded_form(monkeypatch):
+    """Latent attention's other form - this step's keys and values expanded per head into temporary
+    pages, windowed attention over them - with windows, learned sinks and shared pages: unequal whole
+    prompts in one step, then portions and decoding over the latent cache those steps left."""
+    from k8s_llm_monitor_amd.models.hybrid import LatentAttention
+
+    calls = []
+    real = LatentAttention._forward_expanded
+    monkeypatch.setattr(LatentAttention, "_forward_expanded", lambda self, *a: calls.append(1) or real(self, *a))
+    monkeypatch.setattr(LatentAttention, "_expand_ok",
+                        lambda self, h, meta: meta.is_prefill and meta.all_fresh and not meta.num_decode)
+    rig = rig_for(FULL, 6)
+    V = FULL["vocab"]
+    t, u = toks(60, V, 4), toks(21, V, 5)
+    wt, wu = O.forward(FULL, rig.w, t), O.forward(FULL, rig.w, u)
+    a = rig.step([("a", t[:45]), ("b", u[:20])])
+    assert len(calls) == 5
+    b = rig.step([("a", t[45:46]), ("b", u[20:])], end=["b"])
+    c = rig.step([("a", t[46:])], end=["a"])
+    assert len(calls) == 5
+    close(torch.cat([a["a"], b["a"], c["a"]]), wt)
+    close(torch.cat([a["b"], b["b"]]), wu)
+
+
 def test_first_tokens_and_single_token_prompt():
     rig = rig_for(FULL, 7)
     for n in (1, 2, 3):
