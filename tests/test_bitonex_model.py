@@ -592,6 +592,22 @@ def test_gpu_latent_whole_prompts_take_the_expanded_form(monkeypatch):
 
 
 @pytest.mark.gpu
+def test_gpu_long_prompt_on_the_matrix_core_paths():
+    """1300 tokens (81 pages, 21 chunks of the linear attention kernel, more than 1024 keys per query)
+    at matrix-core sizes in bf16: the whole prompt in one step (latent attention in its expanded
+    form), and cut so that the second portion and the decoded tokens read the caches."""
+    cfg = make_cfg([att(4, 2, 128, 128, 64, 1e5, 0.09, mlp=dense(96)), lin(2, 64, 64, (0.95, 0.999)),
+                    lat(4, 96, 32, 128, 48, 64, 0.09, 1e4, mlp=dense(64)), lat(2, 32, 32, 64, 40, 64, 0.12, 1e4, kv_from=2)],
+                   width=128, vocab=211, mult=0.35)
+    cfg["max_positions"] = 2048
+    rig = rig_for(cfg, 7, device="cuda", dtype=torch.bfloat16, num_blocks=96)
+    t = toks(1300, cfg["vocab"], 4)
+    want = O.forward(cfg, rig.w, t)
+    close_most(rig.run_cut("a", t, [1300]), want, 0.05, frac=1.0)
+    close_most(rig.run_cut("a", t, [1100, 190]), want, 0.05, frac=1.0)
+
+
+@pytest.mark.gpu
 def test_gpu_latent_expanded_form_fp32(monkeypatch):
     calls = _force_expanded(monkeypatch)
     cfg = make_cfg([lat(3, 5, 6, 3, 9, 7, 0.4, mlp=dense(13)), att(), lat(5, 3, 6, 7, 5, 7, 0.3, kv_from=0),
