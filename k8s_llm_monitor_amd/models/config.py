@@ -148,12 +148,19 @@ class MoESpec:
     """Routed feed-forward: ``experts`` experts of width ``ff`` of which each token takes ``top``,
     plus an optional shared expert of width ``shared_ff`` (0 = none).  How the router weighs the
     chosen experts, the experts' form and the shared expert's gate belong to the design
-    (DESIGN_TRAITS ``ffn``)."""
+    (DESIGN_TRAITS ``ffn``).  Designs whose experts clamp their pre-activations read ``limit``;
+    designs whose router chooses within the best of ``groups`` equal groups of neighbouring experts
+    read ``groups`` / ``keep_groups`` (1 group: no restriction) and scale the chosen weights by
+    ``route_scale``."""
 
     experts: int
     top: int
     ff: int
     shared_ff: int = 0
+    limit: float = 0.0
+    groups: int = 1
+    keep_groups: int = 1
+    route_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -178,6 +185,12 @@ class LayerSpec:
     def m(self) -> dict:
         return dict(self.mixer)
 
+    def sub(self, prefix: str, kind: str) -> "LayerSpec":
+        """The spec of a mixer nested in this one: the constants under ``prefix.`` (a composite
+        mixer's ``left`` / ``right``), without the prefix, as a layer of ``kind``."""
+        n = len(prefix) + 1
+        return LayerSpec(kind, tuple((k[n:], v) for k, v in self.mixer if k.startswith(prefix + ".")))
+
 
 @dataclass(frozen=True)
 class HybridConfig:
@@ -195,6 +208,8 @@ class HybridConfig:
     logit_scale: float = 1.0
     residual_mult: float = 1.0  # every sublayer's result is scaled by this before it joins the stream
     logit_softcap: float = 0.0  # > 0: logits <- cap * tanh(logits / cap)
+    embed_scale: float = 1.0  # the token embedding is multiplied by this
+    side_dim: int = 0  # > 0: every layer also reads its own slice of a second token table (``side.embed``)
     loop: Optional[tuple] = None  # (start, stop, times): layers start .. stop-1 run `times` times
     bos_id: int = 1
     eos_ids: tuple = (2,)
@@ -252,6 +267,13 @@ class HybridConfig:
 #   latent         what the design fixes for latent attention: ``rotary`` "half" (entry i turns with
 #                  i + n/2) / "pairs" (2i with 2i + 1), ``sink`` True (a learned logit per head in the
 #                  softmax denominator) / False
+#   norm           "rms" / "layer": block and final norms are RMSNorms, or layer norms with a weight
+#                  and no bias ((x - mean) / sqrt(variance + eps) * w)
+#   composite      config ``type`` -> {"left": (MIXERS entry, options), "right": (MIXERS entry, options)}:
+#                  a layer of that type runs two mixers side by side on the same normed input (their
+#                  constants under ``mixer.left`` / ``mixer.right``, tensors under ``mix.left.`` /
+#                  ``mix.right.``) and adds ``left_scale * left + right_scale * right``.  The options
+#                  are what the design fixes for that mixer (models/hybrid.py documents each mixer's)
 DESIGN_TRAITS = {
     "dunesun": dict(block="parallel", one_plus_norm=True, learned_pos=True, token_shift=False,
                     depth_average=False, ffn="swiglu_topk", max_position=2048),
@@ -261,6 +283,16 @@ DESIGN_TRAITS = {
                     depth_average=False, ffn="gated_gelu", max_position=1 << 17, scalar_norm=True,
                     gated_residual=True, mixers={"attention": "rotary_attention"},
                     latent=dict(rotary="pairs", sink=False)),
+    "levovik": dict(block="sequential", one_plus_norm=False, learned_pos=False, token_shift=False,
+                    depth_average=False, ffn="relu_glu_grouped", max_position=1 << 17, norm="layer",
+                    composite={
+                        "parallel": dict(
+                            left=("rotary_attention", dict(rotary="half", qk_norm="after", sink=True, temp=False, gate=False)),
+                            right=("gated_delta", {})),
+                        "parallel_2": dict(
+                            left=("rotary_attention", dict(rotary="pairs", qk_norm="before", values="keys", temp=False,
+                                                           gate=False)),
+                            right=("gated_linear", {}))}),
 }
 
 
@@ -277,9 +309,9 @@ def _flat(d: dict, prefix: str = "") -> list:
 def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig:
     """A :class:`HybridConfig` from a layer-list ``config.json``: ``architecture``, ``vocab``,
     ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``logit_softcap``, ``residual_mult``,
-    ``loop`` {start, stop, times} and
-    ``layers`` [{type, mixer {...}, mlp {kind: moe, expert.ff, router.experts, router.top, shared.ff}
-    | {kind: dense, ff} | null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
+    ``embedding.scale``, ``token_side.dim``, ``loop`` {start, stop, times} and
+    ``layers`` [{type, mixer {...}, mlp {kind: moe, expert.ff, expert.limit, router.experts, router.top,
+    router.scale, router.groups {count, keep}, shared.ff} | {kind: dense, ff} | null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
     arch = str(c["architecture"]).lower()
     if arch not in DESIGN_TRAITS:
         raise ValueError(f"unknown architecture {c['architecture']!r} (known: {sorted(DESIGN_TRAITS)})")
@@ -291,8 +323,12 @@ def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig
             kind = ml.get("kind", "moe")
             if kind == "moe":
                 sh = ml.get("shared")
-                moe = MoESpec(experts=int(ml["router"]["experts"]), top=int(ml["router"]["top"]),
-                              ff=int(ml["expert"]["ff"]), shared_ff=int(sh["ff"]) if sh else 0)
+                rt = ml["router"]
+                gr = rt.get("groups") or {}
+                moe = MoESpec(experts=int(rt["experts"]), top=int(rt["top"]),
+                              ff=int(ml["expert"]["ff"]), shared_ff=int(sh["ff"]) if sh else 0,
+                              limit=float(ml["expert"].get("limit", 0.0)), groups=int(gr.get("count", 1)),
+                              keep_groups=int(gr.get("keep", gr.get("count", 1))), route_scale=float(rt.get("scale", 1.0)))
             elif kind == "dense":
                 moe = DenseSpec(ff=int(ml["ff"]))
             else:
@@ -309,6 +345,8 @@ def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig
                         norm_eps=float(c["norm"]["eps"]), logit_scale=float(c.get("logit_scale", 1.0)),
                         residual_mult=float(c.get("residual_mult", 1.0)),
                         logit_softcap=float(c.get("logit_softcap") or 0.0), loop=loop,
+                        embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                        side_dim=int((c.get("token_side") or {}).get("dim", 0)),
                         bos_id=int(c.get("bos_id", min(1, V - 1))), eos_ids=tuple(c.get("eos_ids", (min(2, V - 1),))))
 
 
@@ -332,6 +370,12 @@ def hybrid_config_to_dict(c: HybridConfig) -> dict:
         elif s.mlp is not None:
             ml = {"kind": "moe", "expert": {"ff": s.mlp.ff}, "router": {"experts": s.mlp.experts, "top": s.mlp.top},
                   "shared": {"ff": s.mlp.shared_ff} if s.mlp.shared_ff else None}
+            if s.mlp.limit:
+                ml["expert"]["limit"] = s.mlp.limit
+            if s.mlp.groups > 1:
+                ml["router"]["groups"] = {"count": s.mlp.groups, "keep": s.mlp.keep_groups}
+            if s.mlp.route_scale != 1.0:
+                ml["router"]["scale"] = s.mlp.route_scale
         layers.append({"type": s.kind, "mixer": nest(s.mixer), "mlp": ml})
     d = {"architecture": c.arch.capitalize(), "vocab": c.vocab_size, "width": c.d_model, "layers": layers,
          "max_positions": c.max_position, "norm": {"eps": c.norm_eps}, "logit_scale": c.logit_scale,
@@ -340,6 +384,10 @@ def hybrid_config_to_dict(c: HybridConfig) -> dict:
         d["residual_mult"] = c.residual_mult
     if c.logit_softcap:
         d["logit_softcap"] = c.logit_softcap
+    if c.embed_scale != 1.0:
+        d["embedding"] = {"scale": c.embed_scale}
+    if c.side_dim:
+        d["token_side"] = {"dim": c.side_dim}
     if c.loop:
         d["loop"] = {"start": c.loop[0], "stop": c.loop[1], "times": c.loop[2]}
     return d

@@ -72,6 +72,11 @@ class _Params:
         self.device, self.dtype, self.seed, self.src, self.empty = device, dtype, seed, src, empty
         self.used: set = set()
 
+    def rows_of(self, name: str, default: int) -> int:
+        """Rows of a tensor whose first size no config key gives (a low-rank bottleneck): the
+        checkpoint's, or ``default`` for a random-init model."""
+        return int(self.src.get(name).shape[0]) if self.src is not None else int(default)
+
     def get(self, name: str, shape: tuple, std: float = 0.02, mean: float = 0.0, small: bool = False) -> torch.Tensor:
         """``small``: a vector or table the kernels read as fp32, kept fp32 on the device."""
         dt = torch.float32 if small else self.dtype
@@ -338,19 +343,33 @@ class LatentAttention:
 
 class RotaryAttention:
     """Grouped-query softmax attention with rotary positions on the first ``rot.dims`` entries of every
-    query / key head (entry i turns with entry i + rot.dims / 2; frequencies ``rot.base^(-2i/dims)``),
-    a learned temperature per query head (``temp``: score = q.k * scale * temp[h]) and a sigmoid
-    output gate ``heads * sigmoid(G h)`` in front of the out-projection.  Causal; ``mask.size`` keys
+    query / key head (frequencies ``rot.base^(-2i/dims)``, optionally rescaled for long contexts by
+    ``rot.scaling`` {factor, low, high, original}, ops.hybrid.rotary_freq).  Causal; ``mask.size`` keys
     of sliding window where given (0 / absent: all).  Pages and attention kernels are windowed
-    attention's; the temperature is folded into the query in the rotation pass.
-    ``tail``: extra rows for the input projection (see LatentAttention)."""
+    attention's.  What a design fixes comes as ``opts`` (absent: the first value):
+
+    * ``rotary`` "half" (entry i turns with entry i + rot.dims / 2) / "pairs" (2i with 2i + 1);
+    * ``temp`` True: a learned temperature per query head (``temp``: score = q.k * scale * temp[h]),
+      folded into the query in the rotation pass;
+    * ``gate`` True: a sigmoid output gate ``heads * sigmoid(G h)`` in front of the out-projection;
+    * ``qk_norm`` None / "before" (every q and k head RMS-normed over ``dim`` with the weights ``q.norm`` /
+      ``k.norm`` [dim], then turned) / "after" (turned, then divided by its root mean square, no weight);
+    * ``sink`` False / True: a learned logit per query head (``sink``) joins the softmax denominator;
+    * ``values`` "own" (``v`` projection) / "keys" (the values are the keys as projected, before norm
+      and turn; no ``v`` tensor, vdim = dim).
+
+    ``tail``: extra rows for the input projection (see LatentAttention).  ``forward(..., proj=)``: the
+    input projection computed by the caller (this mixer's columns of a wider GEMM)."""
 
     kind = "rotary_attention"
 
     def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
-                 tail: Optional[torch.Tensor] = None):
+                 tail: Optional[torch.Tensor] = None, opts: Optional[dict] = None):
         m = spec.m
-        self.H, self.G, self.dk, self.dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+        o = opts or {}
+        self.H, self.G, self.dk = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
+        self.v_from_k = o.get("values", "own") == "keys"
+        self.dv = self.dk if self.v_from_k else int(m["vdim"])
         if self.H % self.G:
             raise ValueError(f"{prefix}: heads {self.H} not a multiple of kv_heads {self.G}")
         self.scale = float(m.get("scale", 1.0 / math.sqrt(self.dk)))
@@ -358,21 +377,31 @@ class RotaryAttention:
         self.base, self.rdims = float(m.get("rot.base", 10000.0)), int(m.get("rot.dims", self.dk))
         if self.rdims % 2 or not 0 <= self.rdims <= self.dk:
             raise ValueError(f"{prefix}: rot.dims {self.rdims} must be even and at most dim {self.dk}")
-        self.pairs = (traits or {}).get("attention_rotary", "half") == "pairs"
+        self.pairs = o.get("rotary", (traits or {}).get("attention_rotary", "half")) == "pairs"
+        self.norm = {None: 0, "before": 1, "after": 2}[o.get("qk_norm")]
+        self.has_temp, self.has_gate, self.sink = bool(o.get("temp", True)), bool(o.get("gate", True)), bool(o.get("sink", False))
+        self.eps = eps
         self.fast = 1
-        nq, nk, nv = self.H * self.dk, self.G * self.dk, self.G * self.dv
+        nq, nk, nv = self.H * self.dk, self.G * self.dk, (0 if self.v_from_k else self.G * self.dv)
         s = 1.0 / math.sqrt(d)
-        ws = [p.get(prefix + "q", (nq, d), s), p.get(prefix + "k", (nk, d), s), p.get(prefix + "v", (nv, d), s),
-              p.get(prefix + "g", (self.H * self.dv, d), s)]
+        ws = [p.get(prefix + "q", (nq, d), s), p.get(prefix + "k", (nk, d), s)]
+        if not self.v_from_k:
+            ws.append(p.get(prefix + "v", (nv, d), s))
+        if self.has_gate:
+            ws.append(p.get(prefix + "g", (self.H * self.dv, d), s))
         self.g_col = nq + nk + nv
-        self.n_in = self.g_col + self.H * self.dv
+        self.n_in = self.g_col + (self.H * self.dv if self.has_gate else 0)
         self.n_tail = 0 if tail is None else tail.shape[0]
         if tail is not None:
             ws.append(tail)
         self.tail_out = None
-        self.w_in = torch.cat(ws).contiguous()  # [q | k | v | gate (| tail)]: one launch
-        self.temp = p.get(prefix + "temp", (self.H,), 0.2, 1.0, small=True)
-        self.freq = hops.rotary_freq(self.base, self.rdims, p.device)
+        self.w_in = torch.cat(ws).contiguous()  # [q | k (| v) (| gate) (| tail)]: one launch
+        self.temp = p.get(prefix + "temp", (self.H,), 0.2, 1.0, small=True) if self.has_temp else None
+        self.qn = p.get(prefix + "q.norm", (self.dk,), 0.1, 1.0, small=True) if self.norm == 1 else None
+        self.kn = p.get(prefix + "k.norm", (self.dk,), 0.1, 1.0, small=True) if self.norm == 1 else None
+        self.sinks = p.get(prefix + "sink", (self.H,), 1.0, small=True) if self.sink else None
+        sc = {k[len("rot.scaling."):]: v for k, v in m.items() if k.startswith("rot.scaling.")}
+        self.freq = hops.rotary_freq(self.base, self.rdims, p.device, scaling=sc or None)
         self.wo = p.get(prefix + "o", (d, self.H * self.dv), 1.0 / math.sqrt(self.H * self.dv))
 
     def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
@@ -382,25 +411,42 @@ class RotaryAttention:
     def cache_bytes(self, esize: int) -> tuple:
         return BLOCK * self.G * (self.dk + self.dv) * esize, 0
 
-    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
         H, G, dk, dv = self.H, self.G, self.dk, self.dv
-        proj = F.linear(h, self.w_in)
+        if proj is None:
+            proj = F.linear(h, self.w_in)
         if self.n_tail:
             self.tail_out = (proj, self.n_in)
         kc, vc = cache["k"], cache["v"]
-        hops.rotary_cache(proj, H, G, dk, dv, meta.positions, self.freq, self.pairs, self.temp, kc, vc, meta.slot_mapping)
-        args = (H, G, dk, dv, self.scale, self.window, False)
+        hops.rotary_cache(proj, H, G, dk, dv, meta.positions, self.freq, self.pairs, self.temp, kc, vc, meta.slot_mapping,
+                          norm=self.norm, qw=self.qn, kw=self.kn, eps=self.eps, v_from_k=self.v_from_k)
+        args = (H, G, dk, dv, self.scale, self.window, self.sink)
         if not meta.is_prefill:
-            o = hops.window_attention_decode(proj, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast))
+            o = hops.window_attention_decode(proj, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast),
+                                             sinks=self.sinks)
         else:
             nd = meta.num_decode
             o = hops.window_attention_prefill(proj[nd:], kc, vc, meta.cu_seqlens, meta.ctx_start, meta.block_tables,
-                                              *args, mfma=self.fast)
+                                              *args, mfma=self.fast, sinks=self.sinks)
             if nd:
                 od = hops.window_attention_decode(proj[:nd], kc, vc, meta.dec_block_tables, meta.dec_seq_lens, *args,
-                                                  vec=bool(self.fast))
+                                                  vec=bool(self.fast), sinks=self.sinks)
                 o = torch.cat([od, o])
-        return F.linear(hops.sigmoid_gate(o, proj, self.g_col), self.wo)
+        if self.has_gate:
+            o = hops.sigmoid_gate(o, proj, self.g_col)
+        return F.linear(o, self.wo)
+
+    def export(self, p: str) -> dict:
+        nq, nk = self.H * self.dk, self.G * self.dk
+        out = {p + "q": self.w_in[:nq], p + "k": self.w_in[nq:nq + nk], p + "o": self.wo}
+        if not self.v_from_k:
+            out[p + "v"] = self.w_in[nq + nk:self.g_col]
+        if self.has_gate:
+            out[p + "g"] = self.w_in[self.g_col:self.n_in]
+        for key, t in (("temp", self.temp), ("q.norm", self.qn), ("k.norm", self.kn), ("sink", self.sinks)):
+            if t is not None:
+                out[p + key] = t
+        return out
 
 
 class LightningMixer:
@@ -456,8 +502,194 @@ class LightningMixer:
         return F.linear(g, self.wo)
 
 
+def _low_rank(p: _Params, prefix: str, name1: str, name2: str, n_out: int, d: int, default: int) -> tuple:
+    """A two-stage projection ``W2 (W1 h)`` whose inner size only the tensors give."""
+    r = p.rows_of(prefix + name1, default)
+    return p.get(prefix + name1, (r, d), 1.0 / math.sqrt(d)), p.get(prefix + name2, (n_out, r), 1.0 / math.sqrt(r))
+
+
+class GatedDeltaMixer:
+    """The delta rule with a decay per head and key channel.  ``q, k`` ([kv_heads, dim]) and ``v``
+    ([heads, vdim]) pass a short causal convolution per channel (``q.conv`` ... [channels, conv taps], no
+    bias) and SiLU; q and k are made unit vectors per head and q is scaled by ``dim^-1/2``;
+    ``beta = sigmoid(W_b h)`` per head; decays ``g = exp(-exp(A_log[h]) softplus(W_a2 (W_a1 h) + dt_bias))``
+    per head and key channel.  Per head (reading q / k head ``h // (heads / kv_heads)``):
+    ``S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q``.  Each head's o is RMS-normed
+    over vdim (weight ``norm`` [vdim], shared by the heads) and multiplied by ``sigmoid(W_g2 (W_g1 h))``,
+    then projected.  State per sequence slot: S (fp32) and the last taps - 1 convolution inputs.
+    Everything behind the convolution is fp32 (ops.hybrid.decay_scan)."""
+
+    kind = "gated_delta"
+    stateful = True
+
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None, opts: Optional[dict] = None):
+        m = spec.m
+        self.H, self.dk, self.dv = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        self.Gk, self.taps = int(m.get("kv_heads", self.H)), int(m["conv"])
+        if self.H % self.Gk or self.taps < 1:
+            raise ValueError(f"{prefix}: heads {self.H} / kv_heads {self.Gk} / conv {self.taps} do not fit")
+        self.eps = eps
+        H, Gk, dk, dv = self.H, self.Gk, self.dk, self.dv
+        s = 1.0 / math.sqrt(d)
+        self.C = 2 * Gk * dk + H * dv  # convolved channels [q | k | v]
+        wa1, self.wa2 = _low_rank(p, prefix, "a1", "a2", H * dk, d, int(m.get("a_rank", 16)))
+        wg1, self.wg2 = _low_rank(p, prefix, "g1", "g2", H * dv, d, int(m.get("g_rank", 16)))
+        self.ra, self.rg = wa1.shape[0], wg1.shape[0]
+        # rows [q | k | v | beta | a1 | g1]: everything that reads the mixer's input, one launch
+        self.w_in = torch.cat([p.get(prefix + "q", (Gk * dk, d), s), p.get(prefix + "k", (Gk * dk, d), s),
+                               p.get(prefix + "v", (H * dv, d), s), p.get(prefix + "b", (H, d), s), wa1, wg1]).contiguous()
+        self.b_col, self.a_col, self.g_col = self.C, self.C + H, self.C + H + self.ra
+        self.conv_w = torch.cat([p.get(prefix + "q.conv", (Gk * dk, self.taps), 0.4, small=True),
+                                 p.get(prefix + "k.conv", (Gk * dk, self.taps), 0.4, small=True),
+                                 p.get(prefix + "v.conv", (H * dv, self.taps), 0.4, small=True)]).contiguous()
+        self.a_log = p.get(prefix + "A_log", (H,), 0.5, -0.5, small=True)
+        self.dt_bias = p.get(prefix + "dt_bias", (H * dk,), 0.5, -1.0, small=True)
+        self.norm_w = p.get(prefix + "norm", (dv,), 0.1, 1.0, small=True)
+        self.norm_all = self.norm_w.repeat(H).contiguous()  # the norm kernel reads one weight per column
+        self.wo = p.get(prefix + "o", (d, H * dv), 1.0 / math.sqrt(H * dv))
+
+    def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
+        return {"conv": torch.zeros(num_slots, max(1, self.taps - 1), self.C, dtype=dtype, device=device),
+                "state": torch.zeros(num_slots, self.H, self.dv, self.dk, dtype=torch.float32, device=device)}
+
+    def cache_bytes(self, esize: int) -> tuple:
+        return 0, (self.taps - 1) * self.C * esize + self.H * self.dk * self.dv * 4
+
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        H, Gk, dk, dv = self.H, self.Gk, self.dk, self.dv
+        if proj is None:
+            proj = F.linear(h, self.w_in)
+        seg = (meta.seg_cu, meta.seg_ctx, meta.seg_slot)
+        qkv = hops.conv_silu(proj, 0, self.C, self.conv_w, None, cache["conv"], *seg)
+        z = F.linear(proj[:, self.a_col:self.a_col + self.ra], self.wa2)
+        gate = F.linear(proj[:, self.g_col:self.g_col + self.rg], self.wg2)
+        o = hops.decay_scan(qkv, 0, Gk * dk, 2 * Gk * dk, z, self.dt_bias, cache["state"], *seg, H, Gk, dk, dv,
+                            dk ** -0.5, a_log=self.a_log, beta=proj, beta_col=self.b_col, unit=True)
+        g = hops.gated_group_norm(o, gate, 0, self.norm_all, self.eps, H, h.dtype, after=True)
+        return F.linear(g, self.wo)
+
+    def export(self, p: str) -> dict:
+        n = self.Gk * self.dk
+        w, cw = self.w_in, self.conv_w
+        return {p + "q": w[:n], p + "k": w[n:2 * n], p + "v": w[2 * n:self.C], p + "b": w[self.b_col:self.a_col],
+                p + "a1": w[self.a_col:self.g_col], p + "g1": w[self.g_col:self.g_col + self.rg], p + "a2": self.wa2,
+                p + "g2": self.wg2, p + "q.conv": cw[:n], p + "k.conv": cw[n:2 * n], p + "v.conv": cw[2 * n:],
+                p + "A_log": self.a_log, p + "dt_bias": self.dt_bias, p + "norm": self.norm_w, p + "o": self.wo}
+
+
+class GatedLinearMixer:
+    """Linear attention with a decay per head and key channel: ``q = W_q h * dim^-1/2``, ``k``, ``v`` per
+    head; ``alpha = sigmoid(W_a2 (W_a1 h) + a2.b)^(1 / tau)``; per head ``S <- diag(alpha) S + k v^T``,
+    ``o = S^T q``.  Each head's o is RMS-normed over vdim (weight ``norm`` [vdim], shared by the heads);
+    the concatenated heads are multiplied by ``silu(W_g h)`` and projected.  The state S is fp32, one
+    per sequence slot (ops.hybrid.decay_scan)."""
+
+    kind = "gated_linear"
+    stateful = True
+
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None, opts: Optional[dict] = None):
+        m = spec.m
+        self.H, self.dk, self.dv, self.tau = int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m.get("tau", 1.0))
+        self.eps = eps
+        H, dk, dv = self.H, self.dk, self.dv
+        s = 1.0 / math.sqrt(d)
+        wa1, self.wa2 = _low_rank(p, prefix, "a1", "a2", H * dk, d, int(m.get("a_rank", 16)))
+        self.ra = wa1.shape[0]
+        # rows [q | k | v | gate | a1]
+        self.w_in = torch.cat([p.get(prefix + "q", (H * dk, d), s), p.get(prefix + "k", (H * dk, d), s),
+                               p.get(prefix + "v", (H * dv, d), s), p.get(prefix + "g", (H * dv, d), s), wa1]).contiguous()
+        self.g_col = 2 * H * dk + H * dv
+        self.a_col = self.g_col + H * dv
+        self.a_bias = p.get(prefix + "a2.b", (H * dk,), 0.5, 3.0, small=True)
+        self.norm_w = p.get(prefix + "norm", (dv,), 0.1, 1.0, small=True)
+        self.norm_all = self.norm_w.repeat(H).contiguous()
+        self.wo = p.get(prefix + "o", (d, H * dv), 1.0 / math.sqrt(H * dv))
+
+    def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
+        return {"state": torch.zeros(num_slots, self.H, self.dv, self.dk, dtype=torch.float32, device=device)}
+
+    def cache_bytes(self, esize: int) -> tuple:
+        return 0, self.H * self.dk * self.dv * 4
+
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        H, dk, dv = self.H, self.dk, self.dv
+        if proj is None:
+            proj = F.linear(h, self.w_in)
+        z = F.linear(proj[:, self.a_col:self.a_col + self.ra], self.wa2)
+        o = hops.decay_scan(proj, 0, H * dk, 2 * H * dk, z, self.a_bias, cache["state"], meta.seg_cu, meta.seg_ctx,
+                            meta.seg_slot, H, H, dk, dv, dk ** -0.5, tau=self.tau)
+        g = hops.gated_group_norm(o, proj, self.g_col, self.norm_all, self.eps, H, h.dtype, after=True, gate="silu")
+        return F.linear(g, self.wo)
+
+    def export(self, p: str) -> dict:
+        n, w = self.H * self.dk, self.w_in
+        return {p + "q": w[:n], p + "k": w[n:2 * n], p + "v": w[2 * n:self.g_col], p + "g": w[self.g_col:self.a_col],
+                p + "a1": w[self.a_col:self.a_col + self.ra], p + "a2": self.wa2, p + "a2.b": self.a_bias,
+                p + "norm": self.norm_w, p + "o": self.wo}
+
+
+class SideBySide:
+    """Two mixers on the same normed input, added with fixed weights: ``left_scale * left(h) +
+    right_scale * right(h)``.  Which two, and what the design fixes for each, is the design's
+    ``composite`` trait for the layer's ``type``; their constants sit under ``mixer.left`` /
+    ``mixer.right`` and their tensors under ``mix.left.`` / ``mix.right.``.  Both input projections run
+    as ONE GEMM (each mixer then reads its own columns); forward returns the two results with their
+    weights, and the sum happens in fp32 in the launch of the next norm (ops.hybrid.sum_norm)."""
+
+    kind = "side_by_side"
+
+    def __init__(self, spec: LayerSpec, d: int, eps: float, p: _Params, prefix: str, traits: Optional[dict] = None,
+                 tail: Optional[torch.Tensor] = None, opts: Optional[dict] = None):
+        comp = (traits or {}).get("composite", {}).get(spec.kind)
+        if comp is None:
+            raise ValueError(f"{prefix}: the design names no pair of mixers for layers of type {spec.kind!r}")
+        m = spec.m
+        self.subs = []
+        for side in ("left", "right"):
+            kind, o = comp[side]
+            self.subs.append(MIXERS[kind](spec.sub(side, kind), d, eps, p, f"{prefix}{side}.", traits=traits, opts=o))
+        self.scales = (float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0)))
+        self.stateful = any(getattr(x, "stateful", False) for x in self.subs)
+        self.n_left = nl = self.subs[0].w_in.shape[0]
+        n = nl + self.subs[1].w_in.shape[0]
+        # rows padded with zeros to a multiple of 8: the kernels' 16-byte accesses need aligned row strides
+        pad = [torch.zeros(-n % 8, d, dtype=self.subs[0].w_in.dtype, device=self.subs[0].w_in.device)] if n % 8 else []
+        self.w_in = torch.cat([x.w_in for x in self.subs] + pad).contiguous()
+        self.subs[0].w_in, self.subs[1].w_in = self.w_in[:nl], self.w_in[nl:n]
+
+    @property
+    def fast(self) -> int:
+        return getattr(self.subs[0], "fast", 1)
+
+    @fast.setter
+    def fast(self, v: int) -> None:
+        for x in self.subs:
+            if hasattr(x, "fast"):
+                x.fast = v
+
+    def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
+        return {"left": self.subs[0].new_cache(num_blocks, num_slots, dtype, device),
+                "right": self.subs[1].new_cache(num_blocks, num_slots, dtype, device)}
+
+    def cache_bytes(self, esize: int) -> tuple:
+        a, b = (x.cache_bytes(esize) for x in self.subs)
+        return a[0] + b[0], a[1] + b[1]
+
+    def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict) -> tuple:
+        proj = F.linear(h, self.w_in)
+        yl = self.subs[0].forward(h, meta, cache["left"], proj=proj[:, :self.n_left])
+        yr = self.subs[1].forward(h, meta, cache["right"], proj=proj[:, self.n_left:self.n_left + self.subs[1].w_in.shape[0]])
+        return (yl, self.scales[0]), (yr, self.scales[1])
+
+    def export(self, p: str) -> dict:
+        return {**self.subs[0].export(p + "left."), **self.subs[1].export(p + "right.")}
+
+
 MIXERS = {WindowAttention.kind: WindowAttention, Mamba2Mixer.kind: Mamba2Mixer, LatentAttention.kind: LatentAttention,
-          RotaryAttention.kind: RotaryAttention, LightningMixer.kind: LightningMixer}
+          RotaryAttention.kind: RotaryAttention, LightningMixer.kind: LightningMixer,
+          GatedDeltaMixer.kind: GatedDeltaMixer, GatedLinearMixer.kind: GatedLinearMixer, SideBySide.kind: SideBySide}
 
 
 class RoutedFFN:
@@ -516,11 +748,13 @@ class DenseFFN:
 
 
 class GatedDenseFFN:
-    """``down(gelu_tanh(gate h) * (up h))``: gate and up (and ``tail``: extra rows whose outputs
-    forward leaves in ``tail_out``) in one projection, the gated unit in one launch."""
+    """``down(act(gate h) * (up h))`` with ``act`` the tanh GELU (or ``relu``, ``silu``): gate and up (and
+    ``tail``: extra rows whose outputs forward leaves in ``tail_out``) in one projection, the gated unit
+    in one launch."""
 
-    def __init__(self, spec: DenseSpec, d: int, p: _Params, prefix: str, tail: Optional[torch.Tensor] = None):
-        self.ff = spec.ff
+    def __init__(self, spec: DenseSpec, d: int, p: _Params, prefix: str, tail: Optional[torch.Tensor] = None,
+                 act: str = "gelu_tanh"):
+        self.ff, self.act = spec.ff, act
         s = 1.0 / math.sqrt(d)
         ws = [p.get(prefix + "gate", (self.ff, d), s), p.get(prefix + "up", (self.ff, d), s)]
         self.n_tail = 0 if tail is None else tail.shape[0]
@@ -534,7 +768,7 @@ class GatedDenseFFN:
         proj = F.linear(h, self.w_in)
         if self.n_tail:
             self.tail_out = (proj, 2 * self.ff)
-        return F.linear(hops.glu(proj, 0, self.ff, "gelu_tanh"), self.w_down)
+        return F.linear(hops.glu(proj, 0, self.ff, self.act), self.w_down)
 
 
 class PlainRoutedFFN:
@@ -566,6 +800,37 @@ class PlainRoutedFFN:
         return hops.moe_experts(h, ids, wts, self.w1, self.w2, shared, None, act="gelu")
 
 
+class GroupRoutedFFN:
+    """Top-k routed gated experts with clamped pre-activations (``g = min(gate_e h, limit)``,
+    ``u = clamp(up_e h, -limit, limit)``, ``down_e(g sigmoid(1.702 g) (u + 1))``).  The fp32 router
+    scores every expert with a sigmoid; the experts form ``groups`` equal groups of neighbours, a
+    group's score is the sum of its two best experts' and only experts of the ``keep_groups`` best groups
+    can be chosen; the chosen scores are divided by their sum and multiplied by ``route_scale``."""
+
+    def __init__(self, spec: MoESpec, d: int, p: _Params, prefix: str):
+        self.E, self.K, self.ff = spec.experts, spec.top, spec.ff
+        self.limit, self.groups, self.keep, self.route_scale = spec.limit, spec.groups, spec.keep_groups, spec.route_scale
+        if not 1 <= self.K <= self.E or self.E % self.groups or not 1 <= self.keep <= self.groups:
+            raise ValueError(f"{prefix}: top {self.K} of {self.E} experts in {self.groups} groups, {self.keep} kept")
+        if self.K > self.keep * (self.E // self.groups):
+            raise ValueError(f"{prefix}: top {self.K} exceeds the experts of {self.keep} groups")
+        if self.limit <= 0:
+            raise ValueError(f"{prefix}: experts of this form need a positive limit")
+        s, s2 = 1.0 / math.sqrt(d), 1.0 / math.sqrt(self.ff)
+        self.il = False
+        # large bf16 steps run on the Mixtral path's tile GEMM (ops.hybrid.moe_experts)
+        self.tile = p.device.type == "cuda" and p.dtype == torch.bfloat16 and self.ff % 128 == 0 and d % 256 == 0
+        self.w13 = torch.stack([torch.cat([p.get(f"{prefix}e{e}.gate", (self.ff, d), s),
+                                           p.get(f"{prefix}e{e}.up", (self.ff, d), s)]) for e in range(self.E)])
+        self.w2 = torch.stack([p.get(f"{prefix}e{e}.down", (d, self.ff), s2) for e in range(self.E)])
+        self.wr = p.get(prefix + "router", (self.E, d), 2 * s, small=True)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ids, wts = hops.moe_router_grouped(h, self.wr, self.E, self.K, self.groups, self.keep, self.route_scale)
+        return hops.moe_experts(h, ids, wts, self.w13, self.w2, None, None, act="clamped_swish", limit=self.limit,
+                                tile=self.tile)
+
+
 def _ffn_for(family: str, spec, d: int, p: _Params, prefix: str, tail: Optional[torch.Tensor] = None):
     """The feed-forward of a layer in a design's family (models/config.DESIGN_TRAITS ``ffn``)."""
     if spec is None:
@@ -574,6 +839,9 @@ def _ffn_for(family: str, spec, d: int, p: _Params, prefix: str, tail: Optional[
         return GatedDenseFFN(spec, d, p, prefix, tail)
     if family == "swiglu_topk" and isinstance(spec, MoESpec):
         return RoutedFFN(spec, d, p, prefix)
+    if family == "relu_glu_grouped":
+        return GatedDenseFFN(spec, d, p, prefix, tail, act="relu") if isinstance(spec, DenseSpec) else \
+            GroupRoutedFFN(spec, d, p, prefix)
     if family == "plain_softmax":
         return DenseFFN(spec, d, p, prefix) if isinstance(spec, DenseSpec) else PlainRoutedFFN(spec, d, p, prefix)
     raise ValueError(f"{prefix}: no {type(spec).__name__} feed-forward in the {family!r} family")
@@ -607,14 +875,28 @@ class HybridLM:
             raise ValueError(f"{cfg.name}: gated residual is not combined with token shift or depth average")
         if self.depth_avg and cfg.loop:
             raise ValueError(f"{cfg.name}: depth average over looped layers is not defined")
+        self.center = tr.get("norm", "rms") == "layer"  # layer norm (weight, no bias) instead of RMSNorm
+        self.composite = bool(tr.get("composite"))
+        self.side_dim = cfg.side_dim
+        # designs whose branches join the stream with weights, through a norm of their own or into a
+        # layer norm take the summing forward (ops.hybrid.sum_norm)
+        self.summed = self.center or self.composite or self.side_dim > 0
+        if self.summed and (self.shifted or self.depth_avg or self.gated or not self.sequential):
+            raise ValueError(f"{cfg.name}: layer norm, side-by-side mixers and per-layer token input are built for "
+                             "plain sequential blocks")
         nm = 1.0 if not self.one_plus else 0.0  # plain norm weights sit around one
         self.embed = p.get("embed", (V, d), 0.5)
         self.pos = p.get("pos", (cfg.max_position, d), 0.1) if tr["learned_pos"] else None
         self.loop_step = p.get("loop.step", (cfg.loop[2], d), 0.1, small=True) if cfg.loop else None
         self.norms, self.norms2, self.mixers, self.ffns, self.shifts, self.dwa = [], [], [], [], [], []
         self.rg1, self.rg2 = [], []  # gated residual: (bias [d] fp32, weight rows kept for export), per sublayer
-        names = tr.get("mixers", {})
+        names = dict(tr.get("mixers", {}))
+        names.update({k: SideBySide.kind for k in tr.get("composite", {})})
         nshape = () if self.scalar_norm else (d,)
+        # per-layer token input: layer i reads columns [i * side_dim, (i + 1) * side_dim) of a second table
+        sd = self.side_dim
+        self.side_embed = p.get("side.embed", (V, len(cfg.layers) * sd), 0.5) if sd else None
+        self.side_gate, self.side_proj, self.side_norm = [], [], []
 
         def norm_w(name):  # one number per norm is kept as a [d] vector: the norm kernels read a vector
             w = p.get(name, nshape, 0.1, nm, small=True)
@@ -637,6 +919,10 @@ class HybridLM:
             self.rg1.append(self._gate_for(self.mixers[-1], g1))
             self.rg2.append(self._gate_for(self.ffns[-1], g2))
             self.norms2.append(norm_w(f"l{i}.norm2") if self.sequential and spec.mlp is not None else None)
+            if sd:
+                self.side_gate.append(p.get(f"l{i}.side.gate", (sd, d), 1.0 / math.sqrt(d)))
+                self.side_proj.append(p.get(f"l{i}.side.proj", (d, sd), 1.0 / math.sqrt(sd)))
+                self.side_norm.append(p.get(f"l{i}.side.norm", (d,), 0.1, 1.0, small=True))
             self.shifts.append(p.get(f"l{i}.shift", (d,), 0.25, 0.4, small=True) if self.shifted else None)
             # depth-average coefficients: random init leans on the newest result so the stream stays sane
             self.dwa.append(p.get(f"l{i}.dwa", (i + 2,), 0.3 / (i + 2), 1.0 / (i + 2), small=True)
@@ -708,12 +994,19 @@ class HybridLM:
         return sum(t.numel() for t in self._tensors())
 
     def _tensors(self) -> list:
-        ts = [self.embed, self.final_norm, self.head] + self.norms
-        ts += [t for t in [self.pos, self.loop_step] + self.norms2 + self.shifts + self.dwa if t is not None]
+        ts = [self.embed, self.final_norm, self.head] + self.norms + self.side_gate + self.side_proj + self.side_norm
+        ts += [t for t in [self.pos, self.loop_step, self.side_embed] + self.norms2 + self.shifts + self.dwa if t is not None]
         ts += [t for g in self.rg1 + self.rg2 if g is not None for t in g.values() if t is not None]
-        for o in self.mixers + [f for f in self.ffns if f is not None]:
+        subs = [x for m in self.mixers for x in getattr(m, "subs", ())]
+        for o in self.mixers + subs + [f for f in self.ffns if f is not None]:
             ts += [v for v in vars(o).values() if isinstance(v, torch.Tensor)]
-        return ts
+        seen, out = set(), []
+        for t in ts:  # a nested mixer's input projection is a view of its parent's: counted once
+            key = (t.untyped_storage().data_ptr(), t.storage_offset(), t.numel())
+            if t._base is None and key not in seen:
+                seen.add(key)
+                out.append(t)
+        return out
 
     # ------------------------------------------------------------------ forward
     def forward(self, ids: torch.Tensor, meta: AttnMeta, caches: list) -> torch.Tensor:
@@ -757,9 +1050,12 @@ class HybridLM:
             stack[1].copy_(stack[0])
             x = stack[1]
         else:
-            x = hops.embed_pos(ids, meta.positions, self.embed, self.pos, meta.dec_src, meta.dec_prev)
+            x = hops.embed_pos(ids, meta.positions, self.embed, self.pos, meta.dec_src, meta.dec_prev,
+                               scale=c.embed_scale)
         if self.gated:
             return self._forward_gated(x, meta, caches)
+        if self.summed:
+            return self._forward_summed(ids, x, meta, caches)
         pending: tuple = ()
         for r, (li, t, first) in enumerate(self.runs):
             if first and self.loop_step is not None:
@@ -784,6 +1080,48 @@ class HybridLM:
             x = x.index_select(0, idx)
             pending = tuple(a.index_select(0, idx) for a in pending)
         hf = hops.add_norm(x, pending, None, self.final_norm, c.norm_eps, self.one_plus, self.dtype)
+        return self._logits(hf)
+
+    def _forward_summed(self, ids: torch.Tensor, x: torch.Tensor, meta: AttnMeta, caches: list) -> torch.Tensor:
+        """Sequential blocks whose branch results join the stream as weighted sums in the launch of
+        the norm that follows (RMS or layer norm).  With a per-layer token input the layer ends with
+        ``y = W_proj (gelu_tanh(W_gate x) * side_embed[token, layer's columns])`` of the finished stream
+        x, joined as ``x += y / rms(y) * side.norm`` - in the next norm's launch too."""
+        c = self.cfg
+        eps, op, ctr, sd = c.norm_eps, self.one_plus, self.center, self.side_dim
+        pend: tuple = ()  # (branch result, weight) pairs not yet in the stream
+        normed = None  # (y, weight vector) of a branch that joins through its own RMS norm
+        for r, (li, t, first) in enumerate(self.runs):
+            if first and self.loop_step is not None:
+                hops.sum_norm(x, pend, normed, None, eps, False, False, torch.float32)  # the stream, complete
+                pend, normed = (), None
+                x += self.loop_step[t]
+            h = hops.sum_norm(x, pend, normed, self.norms[li], eps, ctr, op, self.dtype)
+            y = self.mixers[li].forward(h, meta, caches[self.kv_run[r]])
+            pend, normed = (y if isinstance(y, tuple) else ((y, 1.0),)), None
+            ff = self.ffns[li]
+            if ff is not None:
+                h2 = hops.sum_norm(x, pend, None, self.norms2[li], eps, ctr, op, self.dtype)
+                pend = ((ff.forward(h2), 1.0),)
+            if sd:
+                xs = hops.sum_norm(x, pend, None, None, eps, False, False, self.dtype)  # the finished stream
+                pend = ()
+                g = hops.gated_lookup(F.linear(xs, self.side_gate[li]), self.side_embed, ids, li * sd, meta.dec_src,
+                                      meta.dec_prev)
+                normed = (F.linear(g, self.side_proj[li]), self.side_norm[li])
+            if self.layer_probe is not None:
+                full = x + sum(a.float() * w for a, w in pend)
+                if normed is not None:
+                    yf = normed[0].float()
+                    full = full + yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * normed[1]
+                self.layer_probe.append(full)
+        if meta.logits_idx is not None:
+            idx = meta.logits_idx
+            x = x.index_select(0, idx)
+            pend = tuple((a.index_select(0, idx), w) for a, w in pend)
+            if normed is not None:
+                normed = (normed[0].index_select(0, idx), normed[1])
+        hf = hops.sum_norm(x, pend, normed, self.final_norm, eps, ctr, op, self.dtype)
         return self._logits(hf)
 
     def _logits(self, hf: torch.Tensor) -> torch.Tensor:
@@ -845,9 +1183,14 @@ def state_dict(model: HybridLM) -> dict:
         out["pos"] = model.pos
     if model.loop_step is not None:
         out["loop.step"] = model.loop_step
+    if model.side_embed is not None:
+        out["side.embed"] = model.side_embed
     for i, (n, m, f) in enumerate(zip(model.norms, model.mixers, model.ffns)):
         p = f"l{i}."
         out[p + "norm1"] = one(n)
+        if model.side_dim:
+            out.update({p + "side.gate": model.side_gate[i], p + "side.proj": model.side_proj[i],
+                        p + "side.norm": model.side_norm[i]})
         if model.norms2[i] is not None:
             out[p + "norm2"] = one(model.norms2[i])
         for key, t in (("shift", model.shifts[i]), ("dwa", model.dwa[i])):
@@ -865,10 +1208,8 @@ def state_dict(model: HybridLM) -> dict:
                 out[p + "mix.sink"] = m.sinks
             if m.kv_from is None:
                 out.update({p + "mix.dkv": m.w_down[m.Q:m.n_down], p + "mix.dkv.norm": m.kn})
-        elif isinstance(m, RotaryAttention):
-            nq, nk, nv = m.H * m.dk, m.G * m.dk, m.G * m.dv
-            out.update({p + "mix.q": m.w_in[:nq], p + "mix.k": m.w_in[nq:nq + nk], p + "mix.v": m.w_in[nq + nk:m.g_col],
-                        p + "mix.g": m.w_in[m.g_col:m.n_in], p + "mix.temp": m.temp, p + "mix.o": m.wo})
+        elif hasattr(m, "export"):
+            out.update(m.export(p + "mix."))
         elif isinstance(m, LightningMixer):
             nv, nk = m.H * m.dv, m.H * m.dk
             out.update({p + "mix.v": m.w_in[:nv], p + "mix.k": m.w_in[nv:nv + nk], p + "mix.q": m.w_in[nv + nk:m.n_act],
@@ -885,6 +1226,11 @@ def state_dict(model: HybridLM) -> dict:
             out.update({p + "mlp.gate": f.w_in[:f.ff], p + "mlp.up": f.w_in[f.ff:2 * f.ff], p + "mlp.down": f.w_down})
         elif isinstance(f, DenseFFN):
             out.update({p + "mlp.up": f.w_up, p + "mlp.down": f.w_down, p + "mlp.act": f.act})
+        elif isinstance(f, GroupRoutedFFN):
+            for e in range(f.E):
+                out[f"{p}mlp.e{e}.gate"], out[f"{p}mlp.e{e}.up"] = f.w13[e, :f.ff], f.w13[e, f.ff:]
+                out[f"{p}mlp.e{e}.down"] = f.w2[e]
+            out[p + "mlp.router"] = f.wr
         elif isinstance(f, PlainRoutedFFN):
             for e in range(f.E):
                 out[f"{p}mlp.e{e}.up"], out[f"{p}mlp.e{e}.down"] = f.w1[e], f.w2[e]

@@ -17,7 +17,8 @@ from .hybrid import HybridLM
 from .llama import CausalLM
 
 # config.arch -> model class
-MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM, "kisutar": HybridLM, "bitonex": HybridLM}
+MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM, "kisutar": HybridLM, "bitonex": HybridLM,
+                 "levovik": HybridLM}
 # layer-list designs by the ``architecture`` value of their config.json (lower case)
 LAYER_LIST_ARCHS = set(DESIGN_TRAITS)
 

@@ -7,7 +7,23 @@
 
 extern "C" {
 int k8sllm_hy_embed_pos(float* out, const int* ids, const int* positions, const void* emb, const void* pos,
-                        const int* src, const int* prev, long T, int d, int vocab, int max_pos, int f32, hipStream_t s);
+                        const int* src, const int* prev, long T, int d, int vocab, int max_pos, float scale, int f32,
+                        hipStream_t s);
+int k8sllm_hy_sum_norm(void* out, float* residual, const void* a0, int t0, float s0, const void* a1, int t1, float s1,
+                       const void* y, int ty, const float* wy, const float* w, long rows, int d, float eps, int center,
+                       int one_plus, int f32, hipStream_t s);
+int k8sllm_hy_gated_lookup(void* out, const void* gate, const void* table, long t_stride, int col, const int* ids,
+                           const int* src, const int* prev, long rows, int n, int vocab, int f32, hipStream_t s);
+int k8sllm_hy_rotary_norm_cache(void* qkv, long stride, long T, int Hq, int G, int dk, int dv, const int* positions,
+                                const float* freq, int nf, int pairs, int norm, const float* qw, const float* kw,
+                                float eps, const float* q_scale, void* k_cache, void* v_cache, const int* slots, int bs,
+                                int v_from_k, int f32, hipStream_t s);
+int k8sllm_hy_decay_scan(float* o, const void* qkv, long stride, int q_col, int k_col, int v_col, const void* z,
+                         long z_stride, const float* z_bias, const float* a_log, float inv_tau, const void* beta,
+                         long b_stride, float* state, const int* cu, const int* ctx, const int* slot, int S, int H, int Gk,
+                         int dk, int dv, float q_scale, int unit, int f32, hipStream_t s);
+int k8sllm_hy_router_grouped(int* ids, float* wts, const void* h, long T, int d, const float* wr, int E, int K,
+                             int groups, int keep, float scale, int f32, hipStream_t s);
 int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const void* a1, int t1, const void* a2,
                        int t2, const float* vec, const float* w, long rows, int d, float eps, int one_plus, int f32,
                        hipStream_t s);
@@ -16,7 +32,8 @@ int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_
 int k8sllm_hy_gated_add_norm(void* out, float* residual, const void* y, int yt, const void* gate, long g_stride,
                              const float* bias, float mult, const float* w, long rows, int d, float eps, int one_plus,
                              int vec, int f32, hipStream_t s);
-int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, int vec, int f32, hipStream_t s);
+int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, float limit, int vec, int f32,
+                  hipStream_t s);
 int k8sllm_hy_activation_cols(void* out, const void* x, long x_stride, long rows, int n, int kind, int vec, int f32,
                               hipStream_t s);
 int k8sllm_hy_sigmoid_gate(void* x, const void* z, long z_stride, long rows, int n, int vec, int f32, hipStream_t s);
@@ -47,7 +64,7 @@ int k8sllm_hy_linear_attn_chunk(float* y, const void* vkq, const float* decay, f
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
                      const float* bias, int E, int K, int rows_w, int over_all, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma,
+                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma, float limit,
                            hipStream_t s);
 int k8sllm_hy_combine(float* out, const void* ys, const int* inv, const float* wts, const void* shared,
                       const float* gate, long T, int K, int d, int f32, hipStream_t s);
@@ -104,7 +121,7 @@ int any_dt(const OptT& t, int64_t numel, const char* n) {  // 0 none, 1 bf16, 2 
   return f ? 2 : 1;
 }
 
-void embed_pos(Tensor out, Tensor ids, Tensor positions, Tensor emb, OptT pos, OptT src, OptT prev) {
+void embed_pos(Tensor out, Tensor ids, Tensor positions, Tensor emb, OptT pos, OptT src, OptT prev, double scale) {
   const int f = act(emb, "embed");
   f32c(out, "out");
   i32c(ids, "ids");
@@ -125,7 +142,7 @@ void embed_pos(Tensor out, Tensor ids, Tensor positions, Tensor emb, OptT pos, O
     TORCH_CHECK(src->numel() >= T && prev->numel() >= 1, "src / prev sizes");
   }
   check(k8sllm_hy_embed_pos(out.data_ptr<float>(), ids.data_ptr<int>(), positions.data_ptr<int>(), emb.data_ptr(),
-                            pos.has_value() ? pos->data_ptr() : nullptr, sp, pp, T, (int)d, (int)emb.size(0), maxp, f, cur()),
+                            pos.has_value() ? pos->data_ptr() : nullptr, sp, pp, T, (int)d, (int)emb.size(0), maxp, (float)scale, f, cur()),
         "embed_pos");
 }
 
@@ -148,8 +165,10 @@ void add_norm(Tensor out, Tensor residual, OptT a0, OptT a1, OptT a2, OptT vec, 
         "add_norm");
 }
 
+// after 0: norm(y * silu(z)) * w;  1: norm(y) * w * sigmoid(z);  2: norm(y) * w * silu(z)
 void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w, double eps, int64_t groups,
-                      bool after) {
+                      int64_t after) {
+  TORCH_CHECK(after >= 0 && after <= 2, "gated_group_norm: mode");
   const int f = act(out, "out");
   same(proj, f, "proj");
   f32c(y, "y");
@@ -161,7 +180,7 @@ void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w
               "gated_group_norm: shapes");
   check(k8sllm_hy_gated_group_norm(out.data_ptr(), y.data_ptr<float>(),
                                    (const char*)proj.data_ptr() + z_col * proj.element_size(), proj.stride(0),
-                                   w.data_ptr<float>(), y.size(0), (int)n, (int)groups, (float)eps, after, f, cur()),
+                                   w.data_ptr<float>(), y.size(0), (int)n, (int)groups, (float)eps, (int)after, f, cur()),
         "gated_group_norm");
 }
 
@@ -192,16 +211,18 @@ void gated_add_norm(Tensor out, Tensor residual, Tensor y, Tensor proj, int64_t 
         "gated_add_norm");
 }
 
-// out [rows, f] = act(proj[:, col : col + f]) * proj[:, col + f : col + 2f]; kind 1 tanh GELU, 3 SiLU
-void glu(Tensor out, Tensor proj, int64_t col, int64_t kind) {
+// out [rows, f] = act(proj[:, col : col + f]) * proj[:, col + f : col + 2f]; kind 1 tanh GELU, 3 SiLU, 4 ReLU,
+// 5 the clamped unit g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)
+void glu(Tensor out, Tensor proj, int64_t col, int64_t kind, double limit) {
   const int f = act(proj, "proj");
   same(out, f, "out");
   TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && out.dim() == 2 && out.is_contiguous() && out.size(0) == proj.size(0),
               "glu: layouts");
   const int64_t n = out.size(1);
-  TORCH_CHECK(col >= 0 && col + 2 * n <= proj.size(1) && (kind == 1 || kind == 3), "glu: columns / kind");
+  TORCH_CHECK(col >= 0 && col + 2 * n <= proj.size(1) && (kind == 1 || kind == 3 || kind == 4 || (kind == 5 && limit > 0)),
+              "glu: columns / kind");
   check(k8sllm_hy_glu(out.data_ptr(), (const char*)proj.data_ptr() + col * proj.element_size(), proj.stride(0), proj.size(0),
-                      (int)n, (int)kind, vec8(proj, col, n), f, cur()),
+                      (int)n, (int)kind, (float)limit, vec8(proj, col, n), f, cur()),
         "glu");
 }
 
@@ -347,22 +368,22 @@ void segs(const Tensor& cu, const Tensor& ctx, const Tensor& slot) {
   TORCH_CHECK(cu.numel() == ctx.numel() + 1 && slot.numel() == ctx.numel(), "segments: cu [R+1], ctx [R], slot [R]");
 }
 
-void conv_silu(Tensor out, Tensor proj, int64_t col0, Tensor cw, Tensor cb, Tensor state, Tensor cu, Tensor ctx,
+void conv_silu(Tensor out, Tensor proj, int64_t col0, Tensor cw, OptT cb, Tensor state, Tensor cu, Tensor ctx,
                Tensor slot) {
   const int f = act(proj, "proj");
   same(out, f, "out");
   same(state, f, "conv_state");
   f32c(cw, "conv_w");
-  f32c(cb, "conv_b");
+  if (cb.has_value()) f32c(*cb, "conv_b");
   segs(cu, ctx, slot);
   const int64_t T = proj.size(0), C = cw.size(0), taps = cw.size(1);
   TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && col0 >= 0 && col0 + C <= proj.size(1), "proj columns");
-  TORCH_CHECK(out.is_contiguous() && out.numel() == T * C && cb.numel() == C, "conv_silu: out / bias");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * C && (!cb.has_value() || cb->numel() == C), "conv_silu: out / bias");
   TORCH_CHECK(state.dim() == 3 && state.is_contiguous() && state.size(2) == C && state.size(1) >= taps - 1 &&
                   (taps == 1 || state.size(1) == taps - 1),
               "conv_state [slots, taps-1, C]");
   check(k8sllm_hy_conv_silu(out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)col0, (int)C, cw.data_ptr<float>(),
-                            cb.data_ptr<float>(), (int)taps, state.data_ptr(), cu.data_ptr<int>(), ctx.data_ptr<int>(),
+                            cb.has_value() ? cb->data_ptr<float>() : nullptr, (int)taps, state.data_ptr(), cu.data_ptr<int>(), ctx.data_ptr<int>(),
                             slot.data_ptr<int>(), (int)ctx.numel(), T, f, cur()),
         "conv_silu");
 }
@@ -493,6 +514,156 @@ void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, OptT bia
         "moe_router");
 }
 
+// addends: any float dtype, contiguous [rows, d]; returns 0 / 1 (bf16) / 2 (fp32)
+void sum_norm(Tensor out, Tensor residual, OptT a0, double s0, OptT a1, double s1, OptT y, OptT wy, OptT w, double eps,
+              bool center, bool one_plus) {
+  const int f = act(out, "out");
+  f32c(residual, "residual");
+  TORCH_CHECK(residual.dim() == 2 && out.is_contiguous() && out.numel() == residual.numel(), "sum_norm: out shape");
+  const int64_t rows = residual.size(0), d = residual.size(1);
+  const int t0 = any_dt(a0, rows * d, "addend 0"), t1 = any_dt(a1, rows * d, "addend 1"), ty = any_dt(y, rows * d, "normed addend");
+  const float *wyp = nullptr, *wp = nullptr;
+  if (ty) {
+    TORCH_CHECK(wy.has_value(), "sum_norm: the normed addend needs its weight");
+    f32c(*wy, "normed addend weight");
+    TORCH_CHECK(wy->numel() == d, "sum_norm: wy [d]");
+    wyp = wy->data_ptr<float>();
+  }
+  if (w.has_value()) {
+    f32c(*w, "w");
+    TORCH_CHECK(w->numel() == d, "sum_norm: w [d]");
+    wp = w->data_ptr<float>();
+  }
+  check(k8sllm_hy_sum_norm(out.data_ptr(), residual.data_ptr<float>(), t0 ? a0->data_ptr() : nullptr, t0, (float)s0,
+                           t1 ? a1->data_ptr() : nullptr, t1, (float)s1, ty ? y->data_ptr() : nullptr, ty, wyp, wp, rows,
+                           (int)d, (float)eps, center, one_plus, f, cur()),
+        "sum_norm");
+}
+
+// out [T, n] = gelu_tanh(gate) * table[id, col : col + n]
+void gated_lookup(Tensor out, Tensor gate, Tensor table, Tensor ids, int64_t col, OptT src, OptT prev) {
+  const int f = act(gate, "gate");
+  same(out, f, "out");
+  same(table, f, "table");
+  i32c(ids, "ids");
+  TORCH_CHECK(gate.dim() == 2 && gate.is_contiguous() && out.is_contiguous() && out.numel() == gate.numel(), "gated_lookup: gate / out");
+  TORCH_CHECK(table.dim() == 2 && table.stride(1) == 1, "gated_lookup: table [V, *]");
+  const int64_t T = gate.size(0), n = gate.size(1);
+  TORCH_CHECK(ids.numel() >= T && col >= 0 && col + n <= table.size(1), "gated_lookup: ids / columns");
+  const int* sp = iptr(src, "src");
+  const int* pp = iptr(prev, "prev");
+  TORCH_CHECK((sp == nullptr) == (pp == nullptr), "src and prev come together");
+  if (sp) {
+    TORCH_CHECK(src->numel() >= T && prev->numel() >= 1, "src / prev sizes");
+  }
+  check(k8sllm_hy_gated_lookup(out.data_ptr(), gate.data_ptr(), table.data_ptr(), table.stride(0), (int)col,
+                               ids.data_ptr<int>(), sp, pp, T, (int)n, (int)table.size(0), f, cur()),
+        "gated_lookup");
+}
+
+// rotary_cache with an RMS norm of every q / k head (norm 1: before the turn, weights qw / kw [dk]; 2: after
+// it, no weight); v_from_k: rows are [q | k | ...] and the value pages take the keys as projected
+void rotary_norm_cache(Tensor qkv, int64_t Hq, int64_t G, int64_t dk, int64_t dv, Tensor positions, Tensor freq, bool pairs,
+                       int64_t norm, OptT qw, OptT kw, double eps, OptT q_scale, OptT k_cache, OptT v_cache, OptT slots,
+                       bool v_from_k) {
+  const int f = act(qkv, "qkv");
+  f32c(freq, "freq");
+  i32c(positions, "positions");
+  const int64_t nq = Hq * dk, nk = G * dk, nv = v_from_k ? 0 : G * dv, T = qkv.size(0);
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= nq + nk + nv, "qkv [T, Hq*dk + G*dk (+ G*dv) (+ more)]");
+  TORCH_CHECK(Hq >= 1 && G >= 1 && positions.numel() >= T && 2 * freq.numel() <= dk && dk <= 1024 && norm >= 0 && norm <= 2 &&
+                  (!v_from_k || dv == dk),
+              "rotary_norm_cache: heads / positions / freq / norm");
+  const float *qs = nullptr, *qwp = nullptr, *kwp = nullptr;
+  if (q_scale.has_value()) {
+    f32c(*q_scale, "q_scale");
+    TORCH_CHECK(q_scale->numel() == Hq, "q_scale [Hq]");
+    qs = q_scale->data_ptr<float>();
+  }
+  if (norm == 1) {
+    TORCH_CHECK(qw.has_value() && kw.has_value(), "rotary_norm_cache: norm weights");
+    f32c(*qw, "qw");
+    f32c(*kw, "kw");
+    TORCH_CHECK(qw->numel() == dk && kw->numel() == dk, "q / k norm weights [dk]");
+    qwp = qw->data_ptr<float>();
+    kwp = kw->data_ptr<float>();
+  }
+  void *kc = nullptr, *vc = nullptr;
+  const int* sp = nullptr;
+  if (k_cache.has_value()) {
+    TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
+    pages(*k_cache, f, nk, "k_cache");
+    vpages(*v_cache, *k_cache, f, G, dv);
+    sp = iptr(slots, "slot_mapping");
+    TORCH_CHECK(slots->numel() >= T, "slot_mapping [T]");
+    kc = k_cache->data_ptr();
+    vc = v_cache->data_ptr();
+  }
+  check(k8sllm_hy_rotary_norm_cache(qkv.data_ptr(), qkv.stride(0), T, (int)Hq, (int)G, (int)dk, (int)dv,
+                                    positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), pairs, (int)norm,
+                                    qwp, kwp, (float)eps, qs, kc, vc, sp, k_cache.has_value() ? (int)k_cache->size(1) : 16,
+                                    v_from_k, f, cur()),
+        "rotary_norm_cache");
+}
+
+// The per-channel-decay recurrence (optionally with the delta rule: beta given); see decay_scan.hip
+void decay_scan(Tensor o, Tensor qkv, int64_t q_col, int64_t k_col, int64_t v_col, Tensor z, Tensor z_bias, OptT a_log,
+                double tau, OptT beta, int64_t beta_col, Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t H,
+                int64_t Gk, int64_t dk, int64_t dv, double q_scale, bool unit) {
+  const int f = act(qkv, "qkv");
+  same(z, f, "z");
+  f32c(o, "o");
+  f32c(z_bias, "z_bias");
+  f32c(state, "state");
+  segs(cu, ctx, slot);
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(H >= 1 && Gk >= 1 && H % Gk == 0 && dk >= 1 && dk <= 256 && dv >= 1 && tau > 0, "decay_scan: sizes (dim <= 256)");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && q_col >= 0 && k_col >= 0 && v_col >= 0 &&
+                  q_col + Gk * dk <= qkv.size(1) && k_col + Gk * dk <= qkv.size(1) && v_col + H * dv <= qkv.size(1),
+              "decay_scan: q / k / v columns");
+  TORCH_CHECK(z.dim() == 2 && z.stride(1) == 1 && z.size(0) == T && z.size(1) == H * dk && z_bias.numel() == H * dk,
+              "decay_scan: z [T, H*dk], z_bias [H*dk]");
+  TORCH_CHECK(o.numel() == T * H * dv, "decay_scan: o [T, H*dv]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dv && state.size(3) == dk, "state [slots, H, dv, dk]");
+  const float* ap = nullptr;
+  if (a_log.has_value()) {
+    f32c(*a_log, "A_log");
+    TORCH_CHECK(a_log->numel() == H, "A_log [H]");
+    ap = a_log->data_ptr<float>();
+  }
+  const void* bp = nullptr;
+  long bstride = 0;
+  if (beta.has_value()) {
+    same(*beta, f, "beta");
+    TORCH_CHECK(beta->dim() == 2 && beta->stride(1) == 1 && beta->size(0) == T && beta_col >= 0 && beta_col + H <= beta->size(1),
+                "decay_scan: beta columns");
+    bp = (const char*)beta->data_ptr() + beta_col * beta->element_size();
+    bstride = beta->stride(0);
+  }
+  check(k8sllm_hy_decay_scan(o.data_ptr<float>(), qkv.data_ptr(), qkv.stride(0), (int)q_col, (int)k_col, (int)v_col,
+                             z.data_ptr(), z.stride(0), z_bias.data_ptr<float>(), ap, (float)(1.0 / tau), bp, bstride,
+                             state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
+                             (int)ctx.numel(), (int)H, (int)Gk, (int)dk, (int)dv, (float)q_scale, unit, f, cur()),
+        "decay_scan");
+}
+
+void moe_router_grouped(Tensor ids, Tensor wts, Tensor h, Tensor wr, int64_t E, int64_t K, int64_t groups, int64_t keep,
+                        double scale) {
+  const int f = act(h, "h");
+  i32c(ids, "ids");
+  f32c(wts, "wts");
+  f32c(wr, "router weight");
+  const int64_t T = h.size(0), d = h.size(1);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && wr.dim() == 2 && wr.size(1) == d && wr.size(0) == E, "router: h [T, d], wr [E, d]");
+  TORCH_CHECK(ids.numel() == T * K && wts.numel() == T * K, "router: outputs");
+  TORCH_CHECK(E <= 256 && K >= 1 && K <= 16 && groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups &&
+                  K <= keep * (E / groups),
+              "router: up to 256 experts, top 16 within the kept groups");
+  check(k8sllm_hy_router_grouped(ids.data_ptr<int>(), wts.data_ptr<float>(), h.data_ptr(), T, (int)d, wr.data_ptr<float>(),
+                                 (int)E, (int)K, (int)groups, (int)keep, (float)scale, f, cur()),
+        "moe_router_grouped");
+}
+
 void moe_align(Tensor ids, int64_t E, Tensor offsets, Tensor sorted_idx, Tensor inv_idx) {
   i32c(ids, "ids");
   i32c(offsets, "offsets");
@@ -507,10 +678,11 @@ void moe_align(Tensor ids, int64_t E, Tensor offsets, Tensor sorted_idx, Tensor 
 
 // y [rows, N] = W[e] a over expert-sorted rows; sorted_idx given: a's row of sorted row r is sorted_idx[r] / div
 // act_code: 0 none, 1 SwiGLU (w = [gate rows ; up rows]), 2 erf GELU
+// 3 the clamped gated unit (w = [gate rows ; up rows], limit)
 void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, int64_t act_code, bool il,
-                  bool mfma) {
-  TORCH_CHECK(act_code >= 0 && act_code <= 2, "grouped_gemm: activation code");
-  const bool swiglu = act_code == 1;
+                  bool mfma, double limit) {
+  TORCH_CHECK(act_code >= 0 && act_code <= 3 && (act_code != 3 || limit > 0), "grouped_gemm: activation code");
+  const bool swiglu = act_code == 1 || act_code == 3;
   const int f = act(a, "a");
   same(y, f, "y");
   same(w, f, "w");
@@ -521,7 +693,7 @@ void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx,
   const int64_t N = swiglu ? w.size(1) / 2 : w.size(1);
   TORCH_CHECK(a.size(1) == Kd && y.size(1) == N && offsets.numel() == E + 1 && (!swiglu || w.size(1) % 2 == 0),
               "grouped_gemm: shapes");
-  TORCH_CHECK(!il || (swiglu && N % 64 == 0), "grouped_gemm: interleaved gate/up needs swiglu and ff % 64 == 0");
+  TORCH_CHECK(!il || (act_code == 1 && N % 64 == 0), "grouped_gemm: interleaved gate/up needs swiglu and ff % 64 == 0");
   const int* sp = iptr(sorted_idx, "sorted_idx");
   if (sp) {
     TORCH_CHECK(sorted_idx->numel() == rows && div >= 1 && a.size(0) * div >= rows, "grouped_gemm: gather index");
@@ -529,7 +701,7 @@ void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx,
     TORCH_CHECK(a.size(0) == rows, "grouped_gemm: a rows");
   }
   check(k8sllm_hy_grouped_gemm(y.data_ptr(), a.data_ptr(), w.data_ptr(), offsets.data_ptr<int>(), sp, (int)div, (int)E,
-                               rows, (int)N, (int)Kd, w.size(1) * Kd, (int)act_code, il, f, mfma, cur()),
+                               rows, (int)N, (int)Kd, w.size(1) * Kd, (int)act_code, il, f, mfma, (float)limit, cur()),
         "grouped_gemm");
 }
 
@@ -718,4 +890,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("latent_prep", &latent_prep);
   m.def("latent_queries", &latent_queries);
   m.def("latent_attention", &latent_attention);
+  m.def("sum_norm", &sum_norm);
+  m.def("gated_lookup", &gated_lookup);
+  m.def("rotary_norm_cache", &rotary_norm_cache);
+  m.def("decay_scan", &decay_scan);
+  m.def("moe_router_grouped", &moe_router_grouped);
 }

@@ -1,5 +1,5 @@
 // Mamba-2 mixer kernels (any sizes; state and recurrence fp32).
-//   conv_silu        causal per-channel convolution + SiLU over a column range of the in-projection,
+//   conv_silu        causal per-channel convolution (bias optional) + SiLU over a column range of the in-projection,
 //                    one thread per (row, channel); the taps-1 inputs before a segment come from the
 //                    sequence's conv state slot (zeros for a sequence that starts in this step)
 //   conv_state_step  advances each segment's conv state slot to the segment's end
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(T* __restrict__ out, con
   }
   const int r = row - cu[s];
   const bool carried = ctx[s] > 0;
-  float acc = cb[c];
+  float acc = cb != nullptr ? cb[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int i = r - (taps - 1) + j;  // offset within the segment of the input under tap j
     float x = 0.f;
@@ -84,7 +84,12 @@ __global__ __launch_bounds__(256) void conv_silu_vec8_kernel(T* __restrict__ out
   }
   const int r = row - cu[s];
   const bool carried = ctx[s] > 0;
-  load8(cb + c, acc);
+  if (cb != nullptr) {
+    load8(cb + c, acc);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  }
   for (int j = 0; j < taps; ++j) {
     const int i = r - (taps - 1) + j;
     if (i >= 0)

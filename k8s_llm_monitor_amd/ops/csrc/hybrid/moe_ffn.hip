@@ -4,9 +4,13 @@
 //                 only, or (over_all) the chosen experts' probabilities in the softmax over all E
 //                 logits, not renormalised; one more row of Wr, if present, gives
 //                 gate = sigmoid(Wr[E] h) (the shared expert's)
+//   router_grouped  sigmoid scores; the experts form equal groups of neighbours, a group scores the sum of its
+//                 two largest, only the `keep` best groups' experts can be chosen; the K largest scores among
+//                 them, weights = score / (sum of the chosen + 1e-20) * scale
 //   grouped_gemm  Y[r] = W[e(r)] A[row(r)] over expert-sorted rows r (offsets / sorted_idx from the
 //                 counting sort), the A rows gathered on load; ACT 1 (SwiGLU): W = [gate rows ; up
-//                 rows] and Y = silu(gate) * up; ACT 2: Y = gelu(W A) (erf form).  64 x 64 tiles, fp32
+//                 rows] and Y = silu(gate) * up; ACT 2: Y = gelu(W A) (erf form); ACT 3: gated like 1 with the clamped unit
+//                 g sigmoid(1.702 g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit).  64 x 64 tiles, fp32
 //                 accumulation.
 //   moe_combine   out[t] = sum_k w[t][k] Y[inv[t*K + k]] + gate[t] * shared[t]   (fp32; no gate: 1)
 #include "hy_common.h"
@@ -113,16 +117,95 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
   }
 }
 
+// Sigmoid router with a choice restricted to the best groups.  One workgroup per token: wave w computes the
+// logits of experts w, w + 4, ... (fp32 weights, h widened), thread 0 scores the groups and picks.
+template <typename T>
+__global__ __launch_bounds__(256) void hy_router_grouped_kernel(int* __restrict__ ids, float* __restrict__ wts,
+                                                                const T* __restrict__ h, int d,
+                                                                const float* __restrict__ wr, int E, int K, int groups,
+                                                                int keep, float scale) {
+  __shared__ float sc[kMaxE];
+  __shared__ float gsc[kMaxE];
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* x = h + t * d;
+  for (int e = wave; e < E; e += 4) {
+    const float* w = wr + (long)e * d;
+    float a = 0.f;
+    for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
+    a = wave_sum(a);
+    if (lane == 0) sc[e] = 1.f / (1.f + expf(-a));
+  }
+  __syncthreads();
+  const int per = E / groups;
+  if (threadIdx.x < groups) {  // a group's score: its two largest scores (one expert per group: its score)
+    float m1 = -1.f, m2 = -1.f;
+    for (int e = threadIdx.x * per; e < (threadIdx.x + 1) * per; ++e) {
+      const float v = sc[e];
+      if (v > m1) {
+        m2 = m1;
+        m1 = v;
+      } else if (v > m2) {
+        m2 = v;
+      }
+    }
+    gsc[threadIdx.x] = per > 1 ? m1 + m2 : m1;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (keep < groups) {  // scores of experts outside the best groups drop below every sigmoid
+      for (int k = 0; k < keep; ++k) {
+        int best = -1;
+        float bv = -INFINITY;
+        for (int g = 0; g < groups; ++g)
+          if (gsc[g] > bv) {
+            bv = gsc[g];
+            best = g;
+          }
+        gsc[best] = -INFINITY;  // marks a kept group
+      }
+    }
+    int sel[kMaxK];
+    float val[kMaxK];
+    float z = 0.f;
+    for (int k = 0; k < K; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e) {
+        if (keep < groups && gsc[e / per] != -INFINITY) continue;
+        bool taken = false;
+        for (int j = 0; j < k; ++j) taken |= sel[j] == e;
+        if (!taken && (best < 0 || sc[e] > bv)) {
+          bv = sc[e];
+          best = e;
+        }
+      }
+      sel[k] = best;
+      val[k] = bv;
+      z += bv;
+    }
+    for (int k = 0; k < K; ++k) {
+      ids[t * K + k] = sel[k];
+      wts[t * K + k] = val[k] / (z + 1e-20f) * scale;
+    }
+  }
+}
+
 constexpr int TM = 64, TN = 64, TK = 16;
 
 __device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+__device__ __forceinline__ float clamped_unit_f(float g, float u, float limit) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g * sigmoid_f(1.702f * g) * (u + 1.f);
+}
 
 template <typename T, int ACT>
 __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y, const T* __restrict__ A,
                                                               const T* __restrict__ W, const int* __restrict__ offsets,
                                                               const int* __restrict__ sorted_idx, int div, int E,
-                                                              int N, int Kd, long w_es, int il) {
-  constexpr bool SWIGLU = ACT == 1;
+                                                              int N, int Kd, long w_es, int il, float limit) {
+  constexpr bool SWIGLU = ACT == 1 || ACT == 3;  // gated: gate rows and up rows
   __shared__ float As[TK][TM + 4];
   __shared__ float Ws[TK][TN + 4];
   __shared__ float Us[SWIGLU ? TK : 1][TN + 4];
@@ -199,7 +282,7 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
         T gq, uq;
         stf(&gq, v);
         stf(&uq, accu[i][j]);
-        v = silu_f(ldf(&gq)) * ldf(&uq);
+        v = ACT == 3 ? clamped_unit_f(ldf(&gq), ldf(&uq), limit) : silu_f(ldf(&gq)) * ldf(&uq);
       } else if (ACT == 2) {  // the projection is rounded to the storage dtype before the activation
         T gq;
         stf(&gq, v);
@@ -223,8 +306,8 @@ __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __rest
                                                                   const bf16_t* __restrict__ W,
                                                                   const int* __restrict__ offsets,
                                                                   const int* __restrict__ sorted_idx, int div, int E,
-                                                                  int N, int Kd, long w_es, int il) {
-  constexpr bool SWIGLU = ACT == 1;
+                                                                  int N, int Kd, long w_es, int il, float limit) {
+  constexpr bool SWIGLU = ACT == 1 || ACT == 3;  // gated: gate rows and up rows
   int e = 0, tile = blockIdx.x, r0 = 0, r1 = 0;
   for (; e < E; ++e) {
     r0 = offsets[e];
@@ -272,7 +355,8 @@ __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __rest
       const int r = r0 + 4 * quad + i;
       if (r >= r1) continue;
       float v = acc[t][i];
-      if (SWIGLU) v = silu_f(bf2f(f2bf(v))) * bf2f(f2bf(accu[t][i]));
+      if (ACT == 3) v = clamped_unit_f(bf2f(f2bf(v)), bf2f(f2bf(accu[t][i])), limit);
+      else if (SWIGLU) v = silu_f(bf2f(f2bf(v))) * bf2f(f2bf(accu[t][i]));
       else if (ACT == 2) v = gelu_erf_f(bf2f(f2bf(v)));
       Y[(long)r * N + n] = f2bf(v);
     }
@@ -315,12 +399,27 @@ int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, i
   return (int)hipGetLastError();
 }
 
+int k8sllm_hy_router_grouped(int* ids, float* wts, const void* h, long T, int d, const float* wr, int E, int K,
+                             int groups, int keep, float scale, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (E > kMaxE || K > kMaxK || K < 1 || groups < 1 || E % groups || keep < 1 || keep > groups ||
+      K > keep * (E / groups))
+    return -1;
+  if (f32)
+    hipLaunchKernelGGL(hy_router_grouped_kernel<float>, dim3(T), dim3(256), 0, s, ids, wts, (const float*)h, d, wr, E, K,
+                       groups, keep, scale);
+  else
+    hipLaunchKernelGGL(hy_router_grouped_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, wts, (const bf16_t*)h, d, wr, E, K,
+                       groups, keep, scale);
+  return (int)hipGetLastError();
+}
+
 // rows: the sorted rows in all (an upper bound of the row tiles is rows / 64 + E)
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma,
+                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma, float limit,
                            hipStream_t s) {
   if (rows <= 0) return 0;
-  if (act < 0 || act > 2) return -1;
+  if (act < 0 || act > 3) return -1;
   const bool swiglu = act == 1;
   if (il && (!swiglu || N % 64)) return -1;
   if (!f32 && mfma && Kd % 32 == 0) {
@@ -328,9 +427,11 @@ int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* off
     const dim3 g16((unsigned)(rows / 16 + E), (unsigned)(few ? (N + 15) / 16 : (N + 63) / 64));
 #define K8SLLM_GM(SW, NT)                                                                                        \
   hipLaunchKernelGGL((hy_grouped_gemm_mfma_kernel<SW, NT>), g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,      \
-                     (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il)
+                     (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il, limit)
     if (swiglu) {
       if (few) K8SLLM_GM(1, 1); else K8SLLM_GM(1, 4);
+    } else if (act == 3) {
+      if (few) K8SLLM_GM(3, 1); else K8SLLM_GM(3, 4);
     } else if (act == 2) {
       if (few) K8SLLM_GM(2, 1); else K8SLLM_GM(2, 4);
     } else {
@@ -342,11 +443,13 @@ int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* off
   const dim3 grid((unsigned)(rows / TM + E), (unsigned)((N + TN - 1) / TN));
 #define K8SLLM_GG(T, SW)                                                                                            \
   hipLaunchKernelGGL((hy_grouped_gemm_kernel<T, SW>), grid, dim3(256), 0, s, (T*)Y, (const T*)A, (const T*)W, offsets, \
-                     sorted_idx, div, E, N, Kd, w_es, il)
+                     sorted_idx, div, E, N, Kd, w_es, il, limit)
   if (f32) {
-    if (swiglu) K8SLLM_GG(float, 1); else if (act == 2) K8SLLM_GG(float, 2); else K8SLLM_GG(float, 0);
+    if (swiglu) K8SLLM_GG(float, 1); else if (act == 3) K8SLLM_GG(float, 3); else if (act == 2) K8SLLM_GG(float, 2);
+    else K8SLLM_GG(float, 0);
   } else {
-    if (swiglu) K8SLLM_GG(bf16_t, 1); else if (act == 2) K8SLLM_GG(bf16_t, 2); else K8SLLM_GG(bf16_t, 0);
+    if (swiglu) K8SLLM_GG(bf16_t, 1); else if (act == 3) K8SLLM_GG(bf16_t, 3); else if (act == 2) K8SLLM_GG(bf16_t, 2);
+    else K8SLLM_GG(bf16_t, 0);
   }
 #undef K8SLLM_GG
   return (int)hipGetLastError();

@@ -12,6 +12,9 @@
 //   norm_gate         out = y / rms(y) * w * sigmoid(z)            (y fp32)
 //   sigmoid_gate      x *= sigmoid(z), in place
 //   softcap           x = cap * tanh(x / cap), in place (fp32 logits)
+//   sum_norm          residual += s0 a0 + s1 a1 + y / rms(y) * wy;  out = RMS or layer norm of it times w
+//                     (or the new residual itself, rounded to the activation dtype)
+//   gated_lookup      out = gelu_tanh(gate) * table[id][col : col + n]
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -20,7 +23,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void embed_pos_kernel(float* __restrict__ out, const int* __restrict__ ids,
                                                         const int* __restrict__ positions, const T* __restrict__ emb,
                                                         const T* __restrict__ pos, const int* __restrict__ src,
-                                                        const int* __restrict__ prev, int d, int vocab, int max_pos) {
+                                                        const int* __restrict__ prev, int d, int vocab, int max_pos,
+                                                        float scale) {
   const long t = blockIdx.x;
   int id = ids[t];
   if (src != nullptr && src[t] >= 0) id = prev[src[t]];
@@ -28,7 +32,7 @@ __global__ __launch_bounds__(256) void embed_pos_kernel(float* __restrict__ out,
   const T* e = emb + (long)id * d;
   const T* p = nullptr;
   if (pos != nullptr) p = pos + (long)min(max(positions[t], 0), max_pos - 1) * d;
-  for (int c = threadIdx.x; c < d; c += 256) out[t * d + c] = ldf(e + c) + (p != nullptr ? ldf(p + c) : 0.f);
+  for (int c = threadIdx.x; c < d; c += 256) out[t * d + c] = ldf(e + c) * scale + (p != nullptr ? ldf(p + c) : 0.f);
 }
 
 template <typename T>
@@ -113,7 +117,8 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(T* __restrict__ o
     ss = block_sum<256>(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
     for (int c = threadIdx.x; c < gs; c += 256)
-      stf(out + row * n + (long)g * gs + c, yr[c] * inv * w[(long)g * gs + c] * sigmoid_f(ldf(zr + c)));
+      stf(out + row * n + (long)g * gs + c,
+          yr[c] * inv * w[(long)g * gs + c] * (after == 2 ? silu_f(ldf(zr + c)) : sigmoid_f(ldf(zr + c))));
     return;
   }
   for (int c = threadIdx.x; c < gs; c += 256) {
@@ -295,9 +300,11 @@ __global__ __launch_bounds__(256) void depth_mix_scalar_kernel(float* __restrict
   stack[(long)(n + 1) * plane + i] = acc + coef[n] * top;
 }
 
-// KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below), 3: SiLU
+// KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below), 3: SiLU,
+// 4: ReLU
 template <int KIND>
 __device__ __forceinline__ float act_f(float z, float a, float b) {
+  if (KIND == 4) return fmaxf(z, 0.f);
   if (KIND == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
   if (KIND == 1) return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
   if (KIND == 3) return z / (1.f + expf(-z));
@@ -325,10 +332,22 @@ __global__ __launch_bounds__(256) void activation_cols_kernel(T* __restrict__ ou
   stf(out + r * n + c, act_f<KIND>(ldf(x + r * x_stride + c), 0.f, 0.f));
 }
 
+// KIND 5: the clamped unit g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit);
+// others: act(gate) * up
+template <int KIND>
+__device__ __forceinline__ float glu_unit(float g, float u, float limit) {
+  if (KIND == 5) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoid_f(1.702f * g) * (u + 1.f);
+  }
+  return act_f<KIND>(g, 0.f, 0.f) * u;
+}
+
 // out [rows, f] = act(gu[:, 0:f]) * gu[:, f:2f], gu's rows g_stride apart
 template <typename T, int KIND>
 __global__ __launch_bounds__(256) void glu_kernel(T* __restrict__ out, const T* __restrict__ gu, long g_stride,
-                                                  long rows, int f, int vec) {
+                                                  long rows, int f, int vec, float limit) {
   const int per = vec ? f / 8 : f;
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= rows * per) return;
@@ -340,11 +359,11 @@ __global__ __launch_bounds__(256) void glu_kernel(T* __restrict__ out, const T* 
     load8(g + 8 * c, a);
     load8(g + f + 8 * c, u);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) a[k] = act_f<KIND>(a[k], 0.f, 0.f) * u[k];
+    for (int k = 0; k < 8; ++k) a[k] = glu_unit<KIND>(a[k], u[k], limit);
     store8(out + r * f + 8 * c, a);
     return;
   }
-  stf(out + r * f + c, act_f<KIND>(ldf(g + c), 0.f, 0.f) * ldf(g + f + c));
+  stf(out + r * f + c, glu_unit<KIND>(ldf(g + c), ldf(g + f + c), limit));
 }
 
 // x [rows, n] (contiguous) *= sigmoid(z[:, 0:n]), z's rows z_stride apart
@@ -389,6 +408,128 @@ __global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, co
   for (long k = i; k < n; ++k) stf(out + k, act_f<KIND>(ldf(x + k), a, b));
 }
 
+// residual += s0 a0 + s1 a1 + y / sqrt(mean(y^2) + eps) * wy, then out = the norm of the new residual times w:
+// center 0 the RMS norm, 1 the layer norm (x - mean) / sqrt(mean((x - mean)^2) + eps), the variance taken
+// from the deviations in a pass of its own (no cancellation).  w == nullptr: out = the new residual,
+// rounded to T.  a0, a1, y: any float dtype (0 = absent), contiguous [rows, d].  One workgroup per row; a
+// thread re-reads only what it wrote itself.
+template <typename T>
+__global__ __launch_bounds__(256) void sum_norm_kernel(T* __restrict__ out, float* __restrict__ residual, const void* a0,
+                                                       int t0, float s0, const void* a1, int t1, float s1,
+                                                       const void* y, int ty, const float* __restrict__ wy,
+                                                       const float* __restrict__ w, int d, float eps, int center,
+                                                       int one_plus) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float* r = residual + row * d;
+  const bool v8 = (d & 7) == 0;
+  const int step = v8 ? 8 : 1;
+  float yinv = 0.f;
+  if (ty) {
+    float ss = 0.f;
+    for (int c = threadIdx.x * step; c < d; c += 256 * step) {
+      if (v8) {
+        float a[8];
+        load8_any(y, ty, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += a[i] * a[i];
+      } else {
+        const float a = ld_any(y, ty, row * d + c);
+        ss += a * a;
+      }
+    }
+    ss = block_sum<256>(ss, red);
+    yinv = 1.0f / sqrtf(ss / (float)d + eps);
+    __syncthreads();  // red is reused below
+  }
+  float sum = 0.f, ssq = 0.f;
+  for (int c = threadIdx.x * step; c < d; c += 256 * step) {
+    if (v8) {
+      float x[8], a[8], g[8];
+      load8(r + c, x);
+      if (t0) {
+        load8_any(a0, t0, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += s0 * a[i];
+      }
+      if (t1) {
+        load8_any(a1, t1, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += s1 * a[i];
+      }
+      if (ty) {
+        load8_any(y, ty, row * d + c, a);
+        load8(wy + c, g);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += a[i] * yinv * g[i];
+      }
+      store8(r + c, x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        sum += x[i];
+        ssq += x[i] * x[i];
+      }
+      if (w == nullptr) store8(out + row * d + c, x);
+    } else {
+      float x = r[c];
+      if (t0) x += s0 * ld_any(a0, t0, row * d + c);
+      if (t1) x += s1 * ld_any(a1, t1, row * d + c);
+      if (ty) x += ld_any(y, ty, row * d + c) * yinv * wy[c];
+      r[c] = x;
+      sum += x;
+      ssq += x * x;
+      if (w == nullptr) stf(out + row * d + c, x);
+    }
+  }
+  if (w == nullptr) return;
+  float mean = 0.f;
+  if (center) {
+    mean = block_sum<256>(sum, red) / (float)d;
+    __syncthreads();
+    ssq = 0.f;
+    for (int c = threadIdx.x * step; c < d; c += 256 * step) {
+      if (v8) {
+        float x[8];
+        load8(r + c, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ssq += (x[i] - mean) * (x[i] - mean);
+      } else {
+        ssq += (r[c] - mean) * (r[c] - mean);
+      }
+    }
+  }
+  ssq = block_sum<256>(ssq, red);
+  const float inv = 1.0f / sqrtf(ssq / (float)d + eps);
+  for (int c = threadIdx.x * step; c < d; c += 256 * step) {
+    if (v8) {
+      float x[8], g[8];
+      load8(r + c, x);
+      load8(w + c, g);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = (x[i] - mean) * inv * (one_plus ? 1.f + g[i] : g[i]);
+      store8(out + row * d + c, x);
+    } else {
+      stf(out + row * d + c, (r[c] - mean) * inv * (one_plus ? 1.f + w[c] : w[c]));
+    }
+  }
+}
+
+// out[t][c] = gelu_tanh(gate[t][c]) * table[id(t)][col + c]; ids resolved as in embed_pos
+template <typename T>
+__global__ __launch_bounds__(256) void gated_lookup_kernel(T* __restrict__ out, const T* __restrict__ gate,
+                                                           const T* __restrict__ table, long t_stride, int col,
+                                                           const int* __restrict__ ids, const int* __restrict__ src,
+                                                           const int* __restrict__ prev, long rows, int n, int vocab) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * n) return;
+  const long t = i / n;
+  const int c = (int)(i - t * n);
+  int id = ids[t];
+  if (src != nullptr && src[t] >= 0) id = prev[src[t]];
+  id = min(max(id, 0), vocab - 1);
+  stf(out + i, act_f<1>(ldf(gate + i), 0.f, 0.f) * ldf(table + (long)id * t_stride + col + c));
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -396,15 +537,15 @@ using namespace k8sllm;
 extern "C" {
 
 int k8sllm_hy_embed_pos(float* out, const int* ids, const int* positions, const void* emb, const void* pos,
-                        const int* src, const int* prev, long T, int d, int vocab, int max_pos, int f32,
+                        const int* src, const int* prev, long T, int d, int vocab, int max_pos, float scale, int f32,
                         hipStream_t s) {
   if (T <= 0) return 0;
   if (f32)
     hipLaunchKernelGGL(embed_pos_kernel<float>, dim3(T), dim3(256), 0, s, out, ids, positions, (const float*)emb,
-                       (const float*)pos, src, prev, d, vocab, max_pos);
+                       (const float*)pos, src, prev, d, vocab, max_pos, scale);
   else
     hipLaunchKernelGGL(embed_pos_kernel<bf16_t>, dim3(T), dim3(256), 0, s, out, ids, positions, (const bf16_t*)emb,
-                       (const bf16_t*)pos, src, prev, d, vocab, max_pos);
+                       (const bf16_t*)pos, src, prev, d, vocab, max_pos, scale);
   return (int)hipGetLastError();
 }
 
@@ -421,7 +562,7 @@ int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const
   return (int)hipGetLastError();
 }
 
-// after 0: group_rms_norm(y * silu(z)) * w;  1: group_rms_norm(y) * w * sigmoid(z)
+// after 0: group_rms_norm(y * silu(z)) * w;  1: group_rms_norm(y) * w * sigmoid(z);  2: ... * silu(z)
 int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_stride, const float* w, long rows,
                                int n, int groups, float eps, int after, int f32, hipStream_t s) {
   if (rows <= 0) return 0;
@@ -449,17 +590,19 @@ int k8sllm_hy_gated_add_norm(void* out, float* residual, const void* y, int yt, 
   return (int)hipGetLastError();
 }
 
-// kind: 1 tanh GELU, 3 SiLU
-int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, int vec, int f32,
+// kind: 1 tanh GELU, 3 SiLU, 4 ReLU, 5 the clamped unit (limit)
+int k8sllm_hy_glu(void* out, const void* gu, long g_stride, long rows, int f, int kind, float limit, int vec, int f32,
                   hipStream_t s) {
   const long n = rows * (vec ? f / 8 : f);
   if (n <= 0) return 0;
   const dim3 g((unsigned)((n + 255) / 256));
-#define K8SLLM_GLU(T, K) hipLaunchKernelGGL((glu_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)gu, g_stride, rows, f, vec)
+#define K8SLLM_GLU(T, K) hipLaunchKernelGGL((glu_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)gu, g_stride, rows, f, vec, limit)
   if (f32) {
-    if (kind == 1) K8SLLM_GLU(float, 1); else if (kind == 3) K8SLLM_GLU(float, 3); else return -1;
+    if (kind == 1) K8SLLM_GLU(float, 1); else if (kind == 3) K8SLLM_GLU(float, 3); else if (kind == 4) K8SLLM_GLU(float, 4);
+    else if (kind == 5) K8SLLM_GLU(float, 5); else return -1;
   } else {
-    if (kind == 1) K8SLLM_GLU(bf16_t, 1); else if (kind == 3) K8SLLM_GLU(bf16_t, 3); else return -1;
+    if (kind == 1) K8SLLM_GLU(bf16_t, 1); else if (kind == 3) K8SLLM_GLU(bf16_t, 3); else if (kind == 4) K8SLLM_GLU(bf16_t, 4);
+    else if (kind == 5) K8SLLM_GLU(bf16_t, 5); else return -1;
   }
 #undef K8SLLM_GLU
   return (int)hipGetLastError();
@@ -548,6 +691,34 @@ int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, fl
     if (kind == 0) K8SLLM_ACT(bf16_t, 0); else if (kind == 1) K8SLLM_ACT(bf16_t, 1); else if (kind == 2) K8SLLM_ACT(bf16_t, 2); else if (kind == 3) K8SLLM_ACT(bf16_t, 3); else return -1;
   }
 #undef K8SLLM_ACT
+  return (int)hipGetLastError();
+}
+
+// t0, t1, ty: 0 absent, 1 bf16, 2 fp32.  w == nullptr: no norm, out = the new residual
+int k8sllm_hy_sum_norm(void* out, float* residual, const void* a0, int t0, float s0, const void* a1, int t1, float s1,
+                       const void* y, int ty, const float* wy, const float* w, long rows, int d, float eps, int center,
+                       int one_plus, int f32, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (f32)
+    hipLaunchKernelGGL(sum_norm_kernel<float>, dim3(rows), dim3(256), 0, s, (float*)out, residual, a0, t0, s0, a1, t1, s1,
+                       y, ty, wy, w, d, eps, center, one_plus);
+  else
+    hipLaunchKernelGGL(sum_norm_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, (bf16_t*)out, residual, a0, t0, s0, a1, t1,
+                       s1, y, ty, wy, w, d, eps, center, one_plus);
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_gated_lookup(void* out, const void* gate, const void* table, long t_stride, int col, const int* ids,
+                           const int* src, const int* prev, long rows, int n, int vocab, int f32, hipStream_t s) {
+  const long tot = rows * n;
+  if (tot <= 0) return 0;
+  const dim3 g((unsigned)((tot + 255) / 256));
+  if (f32)
+    hipLaunchKernelGGL(gated_lookup_kernel<float>, g, dim3(256), 0, s, (float*)out, (const float*)gate,
+                       (const float*)table, t_stride, col, ids, src, prev, rows, n, vocab);
+  else
+    hipLaunchKernelGGL(gated_lookup_kernel<bf16_t>, g, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)gate,
+                       (const bf16_t*)table, t_stride, col, ids, src, prev, rows, n, vocab);
   return (int)hipGetLastError();
 }
 }

@@ -9,9 +9,80 @@
 //                  rounding to the activation dtype.  The keys (after the turn) and the values go to the
 //                  pages at slots[t] (< 0: not written): keys [blocks][bs][G*dk], values dim-major
 //                  [blocks][G][dv][bs].
+//   rotary_norm_cache  the same turn with an RMS norm of every query and key head over its dk entries
+//                  (fp32, eps inside the root): norm == 1 before the turn, times qw / kw [dk]; norm == 2 after
+//                  the turn, no weight; norm == 0 none.  v_from_k: the row has no value columns and the value
+//                  pages take the keys as projected (before norm and turn; dv == dk).  One wave per head, the
+//                  head staged in LDS as fp32; the result is rounded to the activation dtype once.
 #include "hy_common.h"
 
 namespace k8sllm {
+
+constexpr int kMaxHeadDim = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ qkv, long stride, int Hq, int G, int dk,
+                                                                int dv, const int* __restrict__ positions,
+                                                                const float* __restrict__ freq, int nf, int pairs,
+                                                                int norm, const float* __restrict__ qw,
+                                                                const float* __restrict__ kw, float eps,
+                                                                const float* __restrict__ q_scale,
+                                                                T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                                const int* __restrict__ slots, int bs, int v_from_k) {
+  extern __shared__ float heads[];  // [4 waves][dk]
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  T* row = qkv + t * stride;
+  const int nq = Hq * dk, nk = G * dk, nv = G * dv;
+  const float pos = (float)positions[t];
+  const long slot = (slots != nullptr && k_cache != nullptr) ? slots[t] : -1;
+  float* x = heads + wave * dk;
+  for (int h0 = 0; h0 < Hq + G; h0 += 4) {  // query heads, then key heads: contiguous in the row
+    // every wave makes every trip (the barriers below are the workgroup's); a wave without a head idles
+    const int h = h0 + wave;
+    const bool live = h < Hq + G;
+    T* hd = row + (long)h * dk;
+    const bool is_k = h >= Hq;
+    const int g = h - Hq;
+    float ss = 0.f;
+    for (int c = lane; live && c < dk; c += 64) {
+      const float v = ldf(hd + c);
+      x[c] = v;
+      ss += v * v;
+      if (is_k && v_from_k && slot >= 0) v_cache[((slot / bs) * nv + (long)g * dv + c) * bs + slot % bs] = hd[c];
+    }
+    if (norm == 1) {
+      const float inv = 1.0f / sqrtf(wave_sum_dpp(ss) / (float)dk + eps);
+      const float* w = is_k ? kw : qw;
+      for (int c = lane; live && c < dk; c += 64) x[c] = x[c] * inv * w[c];
+    }
+    __syncthreads();  // a lane turns pairs whose entries other lanes staged
+    for (int i = lane; live && i < nf; i += 64) {
+      const int a = pairs ? 2 * i : i, b = pairs ? 2 * i + 1 : i + nf;
+      float sn, cs;
+      sincosf(pos * freq[i], &sn, &cs);
+      const float u = x[a], v = x[b];
+      x[a] = u * cs - v * sn;
+      x[b] = v * cs + u * sn;
+    }
+    __syncthreads();
+    float mul = 1.f;
+    if (norm == 2) {
+      float s2 = 0.f;
+      for (int c = lane; live && c < dk; c += 64) s2 += x[c] * x[c];
+      mul = 1.0f / sqrtf(wave_sum_dpp(s2) / (float)dk + eps);
+    }
+    if (live && !is_k && q_scale != nullptr) mul *= q_scale[h];
+    T* kp = (live && is_k && slot >= 0) ? k_cache + slot * (long)nk + (long)g * dk : nullptr;
+    for (int c = lane; live && c < dk; c += 64) {
+      stf(hd + c, x[c] * mul);
+      if (kp != nullptr) kp[c] = hd[c];
+    }
+    __syncthreads();  // the next head reuses x
+  }
+  if (!v_from_k && slot >= 0)
+    for (int c = threadIdx.x; c < nv; c += 256) v_cache[((slot / bs) * nv + c) * bs + slot % bs] = row[nq + nk + c];
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void rotary_cache_kernel(T* __restrict__ qkv, long stride, int Hq, int G, int dk,
@@ -84,6 +155,26 @@ int k8sllm_hy_rotary_cache(void* qkv, long stride, long T, int Hq, int G, int dk
   else
     hipLaunchKernelGGL(rotary_cache_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)qkv, stride, Hq, G, dk, dv,
                        positions, freq, nf, pairs, rot_off, rot_k, q_scale, (bf16_t*)k_cache, (bf16_t*)v_cache, slots, bs);
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_rotary_norm_cache(void* qkv, long stride, long T, int Hq, int G, int dk, int dv, const int* positions,
+                                const float* freq, int nf, int pairs, int norm, const float* qw, const float* kw,
+                                float eps, const float* q_scale, void* k_cache, void* v_cache, const int* slots, int bs,
+                                int v_from_k, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (nf < 0 || 2 * nf > dk || Hq < 1 || G < 1 || dk > kMaxHeadDim || norm < 0 || norm > 2) return -1;
+  if (norm == 1 && (qw == nullptr || kw == nullptr)) return -1;
+  if (v_from_k && dv != dk) return -1;
+  const size_t lds = 4 * (size_t)dk * sizeof(float);
+  if (f32)
+    hipLaunchKernelGGL(rotary_norm_cache_kernel<float>, dim3(T), dim3(256), lds, s, (float*)qkv, stride, Hq, G, dk, dv,
+                       positions, freq, nf, pairs, norm, qw, kw, eps, q_scale, (float*)k_cache, (float*)v_cache, slots, bs,
+                       v_from_k);
+  else
+    hipLaunchKernelGGL(rotary_norm_cache_kernel<bf16_t>, dim3(T), dim3(256), lds, s, (bf16_t*)qkv, stride, Hq, G, dk, dv,
+                       positions, freq, nf, pairs, norm, qw, kw, eps, q_scale, (bf16_t*)k_cache, (bf16_t*)v_cache, slots,
+                       bs, v_from_k);
   return (int)hipGetLastError();
 }
 }

@@ -24,6 +24,7 @@ direction the PV products read along).
 from __future__ import annotations
 
 import importlib
+import math
 from typing import Optional
 
 import torch
@@ -63,14 +64,16 @@ def _silu(z: torch.Tensor) -> torch.Tensor:
 
 def embed_pos(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, pos: Optional[torch.Tensor],
               src: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp32 rows ``embed[id] + pos[position]`` (``pos`` None: no learned positions).  ``src`` /
+              out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """fp32 rows ``embed[id] * scale + pos[position]`` (``pos`` None: no learned positions).  ``src`` /
     ``prev`` (pipelined decode): row i takes token ``prev[src[i]]`` where ``src[i] >= 0``.
     ``out``: a contiguous fp32 [T, d] buffer to fill."""
     if not embed.is_cuda:
         if src is not None:
             ids = torch.where(src >= 0, prev.index_select(0, src.clamp(min=0).long()), ids)
         x = embed[ids.long()].float()
+        if scale != 1.0:
+            x = x * scale
         x = x + pos[positions.long()].float() if pos is not None else x
         if out is not None:
             out.copy_(x)
@@ -78,7 +81,7 @@ def embed_pos(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, p
         return x
     if out is None:
         out = torch.empty(ids.numel(), embed.shape[1], dtype=torch.float32, device=embed.device)
-    native().embed_pos(out, ids, positions, embed, pos, src, prev)
+    native().embed_pos(out, ids, positions, embed, pos, src, prev, float(scale))
     return out
 
 
@@ -100,6 +103,51 @@ def add_norm(residual: torch.Tensor, addends: tuple, vec: Optional[torch.Tensor]
     out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
     a = list(addends) + [None] * (3 - len(addends))
     native().add_norm(out, residual, a[0], a[1], a[2], vec, w, float(eps), bool(one_plus))
+    return out
+
+
+def sum_norm(residual: torch.Tensor, addends: tuple, normed: Optional[tuple], w: Optional[torch.Tensor], eps: float,
+             center: bool, one_plus: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """``residual`` (fp32 [T, d], updated in place) += sum of ``scale * a`` over ``addends`` (at most
+    two (a [T, d] of any float dtype, scale) pairs) + ``y / sqrt(mean(y^2) + eps) * wy`` for ``normed``
+    = (y [T, d], wy [d] fp32) - a branch that joins the stream through an RMS norm of its own.  Returns
+    the norm of the new residual times ``w`` (``one_plus``: ``1 + w``) in ``out_dtype``: ``center`` False
+    the RMS norm, True the layer norm ``(x - mean) / sqrt(mean((x - mean)^2) + eps)``.  ``w`` None: no
+    norm, the new residual itself in ``out_dtype``.  Sums and norms are fp32."""
+    if not residual.is_cuda:
+        for a, sc in addends:
+            residual += a.float() * sc if sc != 1.0 else a.float()
+        if normed is not None:
+            y = normed[0].float()
+            residual += y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * normed[1].float()
+        if w is None:
+            return residual.to(out_dtype)
+        x = residual - residual.mean(-1, keepdim=True) if center else residual
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        wf = w.float()
+        return (h * (1.0 + wf if one_plus else wf)).to(out_dtype)
+    assert len(addends) <= 2
+    out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    a = list(addends) + [(None, 1.0)] * (2 - len(addends))
+    yn, wy = normed if normed is not None else (None, None)
+    native().sum_norm(out, residual, a[0][0], float(a[0][1]), a[1][0], float(a[1][1]), yn, wy, w, float(eps), bool(center),
+                      bool(one_plus))
+    return out
+
+
+def gated_lookup(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col: int,
+                 src: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``gelu_tanh(gate) * table[id, col : col + n]`` for ``gate`` [T, n]: a per-token table slice gated
+    by a projection of the stream (fp32 arithmetic, result in the gate's dtype).  ``src`` / ``prev``: as
+    in embed_pos."""
+    n = gate.shape[1]
+    if not gate.is_cuda:
+        if src is not None:
+            ids = torch.where(src >= 0, prev.index_select(0, src.clamp(min=0).long()), ids)
+        e = table[ids.long(), col:col + n].float()
+        return (F.gelu(gate.float(), approximate="tanh") * e).to(gate.dtype)
+    out = torch.empty_like(gate)
+    native().gated_lookup(out, gate, table, ids, int(col), src, prev)
     return out
 
 
@@ -172,7 +220,7 @@ def depth_mix(stack: torch.Tensor, n: int, addend: Optional[torch.Tensor], coef:
     return stack[n + 1]
 
 
-ACTS = {"gelu": 0, "gelu_tanh": 1, "xielu": 2, "silu": 3}
+ACTS = {"gelu": 0, "gelu_tanh": 1, "xielu": 2, "silu": 3, "relu": 4, "clamped_swish": 5}
 
 
 def _act_torch(z: torch.Tensor, kind: str) -> torch.Tensor:
@@ -182,7 +230,17 @@ def _act_torch(z: torch.Tensor, kind: str) -> torch.Tensor:
         return F.gelu(z, approximate="tanh")
     if kind == "silu":
         return _silu(z)
+    if kind == "relu":
+        return torch.relu(z)
     raise ValueError(kind)
+
+
+def _clamped_unit(g: torch.Tensor, u: torch.Tensor, limit: float) -> torch.Tensor:
+    """Experts with clamped pre-activations: g <- min(g, limit), u <- clamp(u, -limit, limit);
+    g * sigmoid(1.702 g) * (u + 1)."""
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
 
 
 def activation(x: torch.Tensor, kind: str, a: float = 0.0, b: float = 0.0) -> torch.Tensor:
@@ -211,14 +269,18 @@ def activation_cols(proj: torch.Tensor, col: int, n: int, kind: str) -> torch.Te
     return out
 
 
-def glu(proj: torch.Tensor, col: int, f: int, kind: str) -> torch.Tensor:
+def glu(proj: torch.Tensor, col: int, f: int, kind: str, limit: float = 0.0) -> torch.Tensor:
     """Gated linear unit ``act(proj[:, col : col + f]) * proj[:, col + f : col + 2 f]`` ([gate | up]
-    columns of a possibly wider projection) with ``kind`` ``gelu_tanh`` or ``silu``; fp32 arithmetic,
-    [T, f] in the activation dtype."""
+    columns of a possibly wider projection) with ``kind`` ``gelu_tanh``, ``silu`` or ``relu``, or
+    ``clamped_swish``: with g = min(gate, limit) and u = clamp(up, -limit, limit),
+    ``g * sigmoid(1.702 g) * (u + 1)``.  fp32 arithmetic, [T, f] in the activation dtype."""
     if not proj.is_cuda:
-        return (_act_torch(proj[:, col:col + f].float(), kind) * proj[:, col + f:col + 2 * f].float()).to(proj.dtype)
+        g, u = proj[:, col:col + f].float(), proj[:, col + f:col + 2 * f].float()
+        if kind == "clamped_swish":
+            return _clamped_unit(g, u, limit).to(proj.dtype)
+        return (_act_torch(g, kind) * u).to(proj.dtype)
     out = torch.empty(proj.shape[0], f, dtype=proj.dtype, device=proj.device)
-    native().glu(out, proj, int(col), ACTS[kind])
+    native().glu(out, proj, int(col), ACTS[kind], float(limit))
     return out
 
 
@@ -269,7 +331,8 @@ def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: fl
 def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positions: torch.Tensor, freq: torch.Tensor,
                  pairs: bool, q_scale: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                  v_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], rot_off: int = 0,
-                 rot_k: bool = True) -> None:
+                 rot_k: bool = True, norm: int = 0, qw: Optional[torch.Tensor] = None, kw: Optional[torch.Tensor] = None,
+                 eps: float = 0.0, v_from_k: bool = False) -> None:
     """In place on the fused rows [T, Hq*dk | Hkv*dk | Hkv*dv | ...]: the first ``2 len(freq)`` entries
     of every query and key head turn by the angle ``position * freq[i]`` (fp32; ``pairs``: entry 2i
     with 2i + 1, else entry i with i + len(freq); rotary_freq); the rest of a head passes.  ``q_scale``
@@ -277,21 +340,32 @@ def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positio
     temperature folded into the query).  Keys (turned) and values go to the paged cache at
     ``slot_mapping`` (< 0: not written).  ``rot_off``: the turning entries are ``rot_off .. rot_off +
     2 len(freq)`` of every head instead of the first; ``rot_k`` False: the keys are taken as they are
-    (turned already) and only written to the pages."""
+    (turned already) and only written to the pages.
+
+    ``norm``: every query and key head is also RMS-normed over its ``dk`` entries (fp32, ``eps`` inside
+    the root) - 1: BEFORE the turn, times ``qw`` / ``kw`` ([dk] fp32, shared by the heads); 2: AFTER the
+    turn, no weight.  ``v_from_k``: there are no value columns; the values are the keys as projected
+    (before norm and turn), ``dv == dk``."""
     nq, nk, nv = Hq * dk, Hkv * dk, Hkv * dv
     if not qkv.is_cuda:
         T = qkv.shape[0]
 
-        def turn(x):
-            x = x.clone()
-            x[..., rot_off:] = _rotate(x[..., rot_off:], positions, freq, pairs)
-            return x
+        def rms(x):
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
 
-        q = turn(qkv[:, :nq].float().view(T, Hq, dk))
+        def turn(x, w):
+            x = x.clone()
+            if norm == 1:
+                x = rms(x) * w.float()
+            x[..., rot_off:] = _rotate(x[..., rot_off:], positions, freq, pairs)
+            return rms(x) if norm == 2 else x
+
+        q = turn(qkv[:, :nq].float().view(T, Hq, dk), qw)
         if q_scale is not None:
             q = q * q_scale.float().view(1, Hq, 1)
+        k_raw = qkv[:, nq:nq + nk].clone()
         k = qkv[:, nq:nq + nk].float().view(T, Hkv, dk)
-        k = turn(k) if rot_k else k
+        k = turn(k, kw) if rot_k else k
         qkv[:, :nq] = q.reshape(T, nq).to(qkv.dtype)
         qkv[:, nq:nq + nk] = k.reshape(T, nk).to(qkv.dtype)
         if k_cache is not None:
@@ -299,7 +373,11 @@ def rotary_cache(qkv: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int, positio
             s = slot_mapping[:T][ok].long()
             k_cache.view(-1, nk)[s] = qkv[ok, nq:nq + nk]
             bs = k_cache.shape[1]
-            v_cache.view(-1, nv, bs)[s // bs, :, s % bs] = qkv[ok, nq + nk:nq + nk + nv]
+            v_cache.view(-1, nv, bs)[s // bs, :, s % bs] = k_raw[ok] if v_from_k else qkv[ok, nq + nk:nq + nk + nv]
+        return
+    if norm or v_from_k:
+        native().rotary_norm_cache(qkv, Hq, Hkv, dk, dv, positions, freq, bool(pairs), int(norm), qw, kw, float(eps), q_scale,
+                                   k_cache, v_cache, slot_mapping, bool(v_from_k))
         return
     native().rotary_cache(qkv, Hq, Hkv, dk, dv, positions, freq, bool(pairs), q_scale, k_cache, v_cache, slot_mapping,
                           int(rot_off), bool(rot_k))
@@ -383,9 +461,19 @@ def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: t
 
 # ---------------------------------------------------------------- latent attention
 
-def rotary_freq(base: float, dims: int, device=None) -> torch.Tensor:
-    """The ``dims / 2`` rotation frequencies base^(-2i/dims) as fp32 (evaluated in float64)."""
+def rotary_freq(base: float, dims: int, device=None, scaling: Optional[dict] = None) -> torch.Tensor:
+    """The ``dims / 2`` rotation frequencies base^(-2i/dims) as fp32 (evaluated in float64).
+    ``scaling`` {factor, low, high, original}: the long-context rescaling of Llama 3.1 - with the
+    wavelength ``l = 2 pi / f``, a frequency stays where ``l < original / high``, becomes ``f / factor``
+    where ``l > original / low``, and in between is ``(1 - s) f / factor + s f`` with
+    ``s = (original / l - low) / (high - low)``."""
     f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
+    if scaling:
+        fac, lo, hi, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        lam = 2.0 * math.pi / f
+        s = (orig / lam - lo) / (hi - lo) if hi != lo else torch.ones_like(f)
+        mid = (1.0 - s) * f / fac + s * f
+        f = torch.where(lam < orig / hi, f, torch.where(lam > orig / lo, f / fac, mid))
     return f.float().to(device) if device is not None else f.float()
 
 
@@ -509,18 +597,19 @@ def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 # ---------------------------------------------------------------- Mamba-2
 
-def conv_silu(proj: torch.Tensor, col0: int, C: int, conv_w: torch.Tensor, conv_b: torch.Tensor,
+def conv_silu(proj: torch.Tensor, col0: int, C: int, conv_w: torch.Tensor, conv_b: Optional[torch.Tensor],
               conv_state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
               seg_slot: torch.Tensor) -> torch.Tensor:
     """Causal per-channel convolution + SiLU over columns [col0, col0 + C) of ``proj`` [T, *];
-    ``conv_w`` [C, taps] (the last tap multiplies the current token), ``conv_b`` [C].  The taps - 1
+    ``conv_w`` [C, taps] (the last tap multiplies the current token), ``conv_b`` [C] (None: no bias).  The taps - 1
     inputs before a segment come from ``conv_state`` [slots, taps - 1, C] (zeros where seg_ctx is
     0), which is then advanced to the segment's end."""
     T = proj.shape[0]
     taps = conv_w.shape[1]
     if not proj.is_cuda:
         out = torch.empty(T, C, dtype=proj.dtype)
-        wt, bf = conv_w.float().t(), conv_b.float()  # [taps, C]
+        wt = conv_w.float().t()  # [taps, C]
+        bf = conv_b.float() if conv_b is not None else torch.zeros(C)
         cul = seg_cu.tolist()
         for s, (c0, slot) in enumerate(zip(seg_ctx.tolist(), seg_slot.tolist())):
             a, b = cul[s], cul[s + 1]
@@ -619,23 +708,86 @@ def linear_attention(vkq: torch.Tensor, decay: torch.Tensor, state: torch.Tensor
     return ssm_scan(vkq, None, 0, None, None, None, state, seg_cu, seg_ctx, seg_slot, H, dv, dk, H, mode if mode < 3 else 0, decay=decay)
 
 
+def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: torch.Tensor,
+               state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor, seg_slot: torch.Tensor, H: int, Gk: int,
+               dk: int, dv: int, q_scale: float, a_log: Optional[torch.Tensor] = None, tau: float = 1.0,
+               beta: Optional[torch.Tensor] = None, beta_col: int = 0, unit: bool = False) -> torch.Tensor:
+    """Linear attention with a decay per head and key channel, optionally with the delta rule, as an
+    fp32 recurrence over each segment.  Per head h (reading query / key head ``h // (H / Gk)``) and token:
+
+        S <- diag(g_t) S                       g_t [dk]: this token's decays
+        delta rule:   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T
+        otherwise:                                  S <- S + k_t v_t^T
+        o_t = S^T q_t
+
+    ``qkv`` [T, *] holds q, k ([Gk*dk] each) and v ([H*dv]) from columns ``q_col``, ``k_col``, ``v_col``
+    on; q is multiplied by ``q_scale``.  ``unit``: q and k heads are first made unit vectors,
+    ``x / sqrt(sum(x^2) + 1e-6)``.  The decays come from ``z`` [T, H*dk] (a projection, activation dtype)
+    and ``z_bias`` [H*dk] fp32:  ``a_log`` [H] given: ``g = exp(-exp(a_log[h]) softplus(z + z_bias))``;
+    else ``g = sigmoid(z + z_bias)^(1 / tau)``.  ``beta`` [T, *] (given = the delta rule): column
+    ``beta_col + h`` holds head h's logit, ``beta_t = sigmoid(logit)``.  ``state`` [slots, H, dv, dk] fp32
+    (a value row's key channels contiguous) is read at a segment's start (zero where seg_ctx is 0) and
+    written back at its end.  Returns o [T, H*dv] fp32.  Decays, unit norms, gates, state, products and
+    sums are fp32."""
+    T = qkv.shape[0]
+    if not qkv.is_cuda:
+        o = torch.zeros(T, H * dv, dtype=torch.float32)
+        rep = H // Gk
+        cul = seg_cu.tolist()
+        for s, (c0, slot) in enumerate(zip(seg_ctx.tolist(), seg_slot.tolist())):
+            a, b = cul[s], cul[s + 1]
+            if slot < 0 or b <= a:
+                continue
+            n = b - a
+            q = qkv[a:b, q_col:q_col + Gk * dk].float().view(n, Gk, dk)
+            k = qkv[a:b, k_col:k_col + Gk * dk].float().view(n, Gk, dk)
+            v = qkv[a:b, v_col:v_col + H * dv].float().view(n, H, dv)
+            if unit:
+                q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6)
+                k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+            q = (q * q_scale).repeat_interleave(rep, dim=1)
+            k = k.repeat_interleave(rep, dim=1)
+            zz = (z[a:b].float() + z_bias.float()).view(n, H, dk)
+            if a_log is not None:
+                g = torch.exp(-torch.exp(a_log.float()).view(1, H, 1) * F.softplus(zz, threshold=30.0))
+            else:
+                g = torch.exp(F.logsigmoid(zz) / tau)
+            bt = torch.sigmoid(beta[a:b, beta_col:beta_col + H].float()) if beta is not None else None
+            S = state[slot].clone() if c0 > 0 else torch.zeros_like(state[slot])  # [H, dv, dk]
+            for t in range(n):
+                S = S * g[t, :, None, :]
+                if bt is not None:
+                    u = bt[t, :, None] * (v[t] - torch.einsum("hpn,hn->hp", S, k[t]))
+                else:
+                    u = v[t]
+                S = S + u[:, :, None] * k[t, :, None, :]
+                o[a + t] = torch.einsum("hpn,hn->hp", S, q[t]).reshape(-1)
+            state[slot] = S
+        return o
+    o = torch.empty(T, H * dv, dtype=torch.float32, device=qkv.device)
+    native().decay_scan(o, qkv, int(q_col), int(k_col), int(v_col), z, z_bias, a_log, float(tau), beta, int(beta_col),
+                        state, seg_cu, seg_ctx, seg_slot, int(H), int(Gk), int(dk), int(dv), float(q_scale), bool(unit))
+    return o
+
+
 def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, w: torch.Tensor, eps: float, groups: int,
-                     out_dtype: torch.dtype, after: bool = False) -> torch.Tensor:
+                     out_dtype: torch.dtype, after: bool = False, gate: str = "sigmoid") -> torch.Tensor:
     """``y`` [T, n] fp32 times silu of the gate ``proj[:, z_col : z_col + n]``, then RMS-normed in
     ``groups`` equal parts (each by its own root mean square) times ``w`` [n].  ``after``: the norm
-    first (of ``y`` as it is), then times ``w`` and the SIGMOID of the gate."""
+    first (of ``y`` as it is), then times ``w`` and the SIGMOID of the gate (``gate`` "silu": its SiLU)."""
     T, n = y.shape
     if not y.is_cuda:
         if after:
             g = y.view(T, groups, n // groups)
             g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
-            return (g.reshape(T, n) * w.float() * torch.sigmoid(proj[:, z_col:z_col + n].float())).to(out_dtype)
+            z = proj[:, z_col:z_col + n].float()
+            return (g.reshape(T, n) * w.float() * (torch.sigmoid(z) if gate == "sigmoid" else _silu(z))).to(out_dtype)
         g = y * _silu(proj[:, z_col:z_col + n].float())
         g = g.view(T, groups, n // groups)
         g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
         return (g.reshape(T, n) * w.float()).to(out_dtype)
     out = torch.empty(T, n, dtype=out_dtype, device=y.device)
-    native().gated_group_norm(out, y, proj, int(z_col), w, float(eps), int(groups), bool(after))
+    native().gated_group_norm(out, y, proj, int(z_col), w, float(eps), int(groups), (2 if gate == "silu" else 1) if after else 0)
     return out
 
 
@@ -665,6 +817,32 @@ def moe_router(h: torch.Tensor, wr: torch.Tensor, bias: Optional[torch.Tensor], 
     return ids, wts, gate
 
 
+def moe_router_grouped(h: torch.Tensor, wr: torch.Tensor, E: int, K: int, groups: int, keep: int,
+                       scale: float) -> tuple:
+    """fp32 router with sigmoid scores and a choice restricted to groups: ``s = sigmoid(wr h)``; the E
+    experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest
+    scores (its one score where a group is one expert), and only experts of the ``keep`` best groups
+    can be chosen; the ``K`` largest scores among those are taken (lowest index wins a tie) and
+    weighted ``s / (sum of the chosen s + 1e-20) * scale``.  Returns (ids [T, K] int32, weights [T, K] fp32)."""
+    T = h.shape[0]
+    if not h.is_cuda:
+        sc = torch.sigmoid(h.float() @ wr.float().t())
+        masked = sc
+        if groups > 1:
+            per = E // groups
+            gs = sc.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+            best = gs.topk(keep, dim=-1).indices
+            ok = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+            masked = torch.where(ok.repeat_interleave(per, dim=1), sc, torch.full_like(sc, -1.0))
+        idx = masked.topk(K, dim=-1).indices
+        w = sc.gather(1, idx)
+        return idx.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    ids = torch.empty(T, K, dtype=torch.int32, device=h.device)
+    wts = torch.empty(T, K, dtype=torch.float32, device=h.device)
+    native().moe_router_grouped(ids, wts, h, wr, int(E), int(K), int(groups), int(keep), float(scale))
+    return ids, wts
+
+
 # expert-sorted rows from which the routed GEMMs of an interleaved (``il``) layer go to the
 # framework's 256 x 256 prefill tile kernel (ops.moe_grouped_gemm) instead of the 16-row kernel
 TILE_MIN_ROWS = 1024
@@ -672,12 +850,14 @@ TILE_MIN_ROWS = 1024
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
                 shared: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, il: bool = False,
-                mfma: bool = True, act: str = "swiglu") -> torch.Tensor:
+                mfma: bool = True, act: str = "swiglu", limit: float = 0.0, tile: bool = False) -> torch.Tensor:
     """Sum over each token's chosen experts of ``wts * down_e(silu(gate_e h) * up_e h)`` with
     ``w13`` [E, 2*ff, d] (gate rows then up rows; ``il``: interleaved per 128 rows as [64 gate |
     64 up], ops.interleave_gate_up) and ``w2`` [E, d, ff], plus ``gate * shared`` (the shared
     expert's output [T, d] and its per-token gate; ``gate`` None: 1).  ``act`` "gelu": ungated
-    experts ``down_e(gelu(up_e h))`` with ``w13`` [E, ff, d].  fp32 [T, d].
+    experts ``down_e(gelu(up_e h))`` with ``w13`` [E, ff, d].  ``act`` "clamped_swish": gated experts whose
+    unit is ``g * sigmoid(1.702 g) * (u + 1)`` with g = min(gate_e h, limit), u = clamp(up_e h, -limit,
+    limit).  fp32 [T, d].
 
     GPU: the (token, slot) pairs are counting-sorted by expert on the device and both projections
     run as ONE grouped launch each over the sorted rows (SwiGLU in the first epilogue); no host
@@ -700,6 +880,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
                 gu = (hf[rows] @ we.t()).to(h.dtype).float()
                 if act == "gelu":
                     a = F.gelu(gu).to(h.dtype).float()
+                elif act == "clamped_swish":
+                    a = _clamped_unit(gu[:, :ff], gu[:, ff:], limit).to(h.dtype).float()
                 else:
                     a = (_silu(gu[:, :ff]) * gu[:, ff:]).to(h.dtype).float()
                 out.index_add_(0, rows, (a @ w2[e].float().t()).to(h.dtype).float() * wts[rows, slot].unsqueeze(-1))
@@ -712,12 +894,18 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
     sorted_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     inv_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     ext.moe_align(ids, E, offsets, sorted_idx, inv_idx)
-    code = {"swiglu": 1, "gelu": 2}[act]
+    code = {"swiglu": 1, "gelu": 2, "clamped_swish": 3}[act]
     if act == "gelu" and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16 and ff % 256 == 0 and d % 256 == 0:
         from .. import ops  # large steps of plain experts: the prefill tile GEMM twice, GELU between
 
         xs = ops.gather_rows(h, sorted_idx, K)
         a = activation(ops.moe_grouped_gemm(xs, w13, offsets, zero_fill=False), "gelu")
+        ys = ops.moe_grouped_gemm(a, w2, offsets, zero_fill=False)
+    elif act == "clamped_swish" and tile and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
+        from .. import ops  # large steps: the prefill tile GEMM twice, the clamped unit as a launch between
+
+        xs = ops.gather_rows(h, sorted_idx, K)
+        a = glu(ops.moe_grouped_gemm(xs, w13, offsets, zero_fill=False), 0, ff, "clamped_swish", limit)
         ys = ops.moe_grouped_gemm(a, w2, offsets, zero_fill=False)
     elif il and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
         from .. import ops  # the Mixtral path's kernels (_k8sllm_ops)
@@ -727,9 +915,9 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
         ys = ops.moe_grouped_gemm(a, w2, offsets, zero_fill=False)
     else:
         a = torch.empty(n, ff, dtype=h.dtype, device=h.device)
-        ext.grouped_gemm(a, h, w13, offsets, sorted_idx, K, code, il, mfma)
+        ext.grouped_gemm(a, h, w13, offsets, sorted_idx, K, code, il, mfma, float(limit))
         ys = torch.empty(n, d, dtype=h.dtype, device=h.device)
-        ext.grouped_gemm(ys, a, w2, offsets, None, 1, 0, False, mfma)
+        ext.grouped_gemm(ys, a, w2, offsets, None, 1, 0, False, mfma, 0.0)
     out = torch.empty(T, d, dtype=torch.float32, device=h.device)
     ext.moe_combine(out, ys, inv_idx, wts, shared, gate)
     return out
