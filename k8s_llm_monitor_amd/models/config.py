@@ -453,3 +453,32 @@ BITONEX_TINY = _reg(HybridConfig(
             _with_mlp(_lightning(2, 24, 40, (0.9, 0.97)), None),
             _with_mlp(_latent(2, 24, 8, 16, 32, 24, 0, 0.18, base=5000.0, kv_from=1), DenseSpec(64))),
     max_position=4096, norm_eps=1e-6, residual_mult=0.4, logit_softcap=20.0, bos_id=1, eos_ids=(2,)))
+
+
+def _pair(kind, left: dict, right: dict, left_scale: float, right_scale: float) -> LayerSpec:
+    """A layer of two mixers side by side (DESIGN_TRAITS ``composite``): nested constants flattened with dots."""
+    m = {"left_scale": left_scale, "right_scale": right_scale}
+    m.update(_flat({"left": left, "right": right}))
+    return LayerSpec(kind, tuple(sorted(m.items())))
+
+
+def _rot(dims, base, factor, original, low=1.0, high=4.0) -> dict:
+    return {"dims": dims, "base": base, "scaling": {"factor": factor, "low": low, "high": high, "original": original}}
+
+
+# Small Levovik-design model for CPU tests and GPU smoke runs (random weights): softmax attention beside
+# gated linear attention (``parallel_2``) and beside the gated delta rule (``parallel``), a dense, two
+# routed and one absent feed-forward, a per-layer token input.
+LEVOVIK_TINY = _reg(HybridConfig(
+    name="levovik-tiny", arch="levovik", vocab_size=352, d_model=96,
+    layers=(_with_mlp(_pair("parallel_2", dict(heads=4, kv_heads=2, dim=16, scale=0.25, rot=_rot(8, 10000.0, 4.0, 64)),
+                            dict(heads=2, dim=24, vdim=16, tau=8.0, a_rank=8), 0.7, 1.2), DenseSpec(144)),
+            _with_mlp(_pair("parallel", dict(heads=3, kv_heads=1, dim=32, vdim=24, scale=0.18, rot=_rot(16, 50000.0, 8.0, 64)),
+                            dict(heads=4, kv_heads=2, dim=16, vdim=24, conv=3, a_rank=12, g_rank=8), 0.9, 0.6),
+                      MoESpec(8, 2, 40, limit=1.25, groups=4, keep_groups=2, route_scale=1.5)),
+            _with_mlp(_pair("parallel_2", dict(heads=2, kv_heads=2, dim=32, scale=0.2, rot=_rot(32, 10000.0, 2.0, 128)),
+                            dict(heads=3, dim=8, vdim=32, tau=4.0), 1.0, 1.0), None),
+            _with_mlp(_pair("parallel", dict(heads=4, kv_heads=4, dim=16, vdim=16, scale=0.25, rot=_rot(4, 1000.0, 4.0, 32)),
+                            dict(heads=2, kv_heads=2, dim=24, vdim=8, conv=4), 0.8, 0.5),
+                      MoESpec(6, 3, 24, limit=2.0, groups=2, keep_groups=1, route_scale=2.5))),
+    max_position=1 << 17, norm_eps=1e-5, logit_scale=0.6, embed_scale=9.0, side_dim=12, bos_id=1, eos_ids=(2,)))

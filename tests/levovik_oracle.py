@@ -240,7 +240,7 @@ def forward(cfg: dict, weights: dict, tokens, layers_out: list | None = None) ->
     w = {k: v.to(F64) if v.is_floating_point() else v for k, v in weights.items()}
     eps = float(cfg["norm"]["eps"])
     tok = torch.as_tensor(tokens, dtype=torch.long)
-    x = w["embed"][tok] * float(cfg["embedding"]["scale"])
+    x = w["embed"][tok] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     side = cfg.get("token_side")
     for i, L in enumerate(cfg["layers"]):
         p = f"l{i}."
@@ -265,3 +265,84 @@ def forward(cfg: dict, weights: dict, tokens, layers_out: list | None = None) ->
             layers_out.append(x.clone())
     hf = layer_norm(x, w["final.norm"], eps)
     return (hf @ w["head"].T) * float(cfg.get("logit_scale", 1.0))
+
+
+def layers_of(cfg: dict, weights: dict, tokens) -> torch.Tensor:
+    """The residual stream after every layer, [layers, T, width]."""
+    out: list = []
+    forward(cfg, weights, tokens, layers_out=out)
+    return torch.stack(out)
+
+
+def greedy(cfg: dict, w: dict, prompt, n: int) -> list:
+    """``n`` tokens by repeated whole-sequence forwards, each the argmax of the last logits."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = int(torch.argmax(forward(cfg, w, seq)[-1]))
+        out.append(t)
+        seq.append(t)
+    return out
+
+
+def random_weights(cfg: dict, seed: int = 0) -> dict:
+    """Random tensors of a config's shapes (values a bf16 checkpoint could hold), by name.  The inner
+    sizes of the two-stage projections are the mixer's ``a_rank`` / ``g_rank`` (absent: 5 and 7)."""
+    g = torch.Generator().manual_seed(seed)
+    d, V = cfg["width"], cfg["vocab"]
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(torch.bfloat16).float()
+
+    w = {"embed": rnd(V, d, std=0.8 / float((cfg.get("embedding") or {}).get("scale", 1.0))),
+         "final.norm": rnd(d, std=0.1, mean=1.0), "head": rnd(V, d, std=2 * d ** -0.5)}
+    sd = int((cfg.get("token_side") or {}).get("dim", 0))
+    if sd:
+        w["side.embed"] = rnd(V, sd * len(cfg["layers"]), std=0.8)
+    for i, spec in enumerate(cfg["layers"]):
+        L, m = f"l{i}.", spec["mixer"]
+        w[L + "norm1"] = rnd(d, std=0.1, mean=1.0)
+        a, b, P, Q = m["left"], m["right"], f"l{i}.mix.left.", f"l{i}.mix.right."
+        H, G, dk = a["heads"], a["kv_heads"], a["dim"]
+        w[P + "q"], w[P + "k"] = rnd(H * dk, d, std=1.5 * d ** -0.5), rnd(G * dk, d, std=1.5 * d ** -0.5)
+        if spec["type"] == "parallel":
+            dv = a["vdim"]
+            w[P + "v"], w[P + "sink"] = rnd(G * dv, d, std=d ** -0.5), rnd(H, std=1.0)
+        else:
+            dv = dk
+            w[P + "q.norm"], w[P + "k.norm"] = rnd(dk, std=0.2, mean=1.0), rnd(dk, std=0.2, mean=1.0)
+        w[P + "o"] = rnd(d, H * dv, std=(H * dv) ** -0.5)
+        H, dk, dv = b["heads"], b["dim"], b["vdim"]
+        ra, rg = int(b.get("a_rank", 5)), int(b.get("g_rank", 7))
+        if spec["type"] == "parallel":
+            Gk, taps = b["kv_heads"], b["conv"]
+            for n, rows in (("q", Gk * dk), ("k", Gk * dk), ("v", H * dv)):
+                w[Q + n], w[Q + n + ".conv"] = rnd(rows, d, std=1.5 * d ** -0.5), rnd(rows, taps, std=0.5)
+            w[Q + "b"] = rnd(H, d, std=2 * d ** -0.5)
+            w[Q + "A_log"], w[Q + "dt_bias"] = rnd(H, std=0.6, mean=-0.5), rnd(H * dk, std=0.7, mean=-1.0)
+            w[Q + "a1"], w[Q + "a2"] = rnd(ra, d, std=d ** -0.5), rnd(H * dk, ra, std=2 * ra ** -0.5)
+            w[Q + "g1"], w[Q + "g2"] = rnd(rg, d, std=d ** -0.5), rnd(H * dv, rg, std=2 * rg ** -0.5)
+        else:
+            for n, rows in (("q", H * dk), ("k", H * dk), ("v", H * dv), ("g", H * dv)):
+                w[Q + n] = rnd(rows, d, std=1.2 * d ** -0.5)
+            w[Q + "a1"], w[Q + "a2"] = rnd(ra, d, std=d ** -0.5), rnd(H * dk, ra, std=2 * ra ** -0.5)
+            w[Q + "a2.b"] = rnd(H * dk, std=1.0, mean=2.0)
+        w[Q + "norm"] = rnd(dv, std=0.1, mean=1.0)
+        w[Q + "o"] = rnd(d, H * dv, std=(H * dv) ** -0.5)
+        ml = spec.get("mlp")
+        if ml is not None:
+            w[L + "norm2"] = rnd(d, std=0.1, mean=1.0)
+            if ml["kind"] == "dense":
+                f = ml["ff"]
+                w[L + "mlp.gate"], w[L + "mlp.up"] = rnd(f, d, std=d ** -0.5), rnd(f, d, std=d ** -0.5)
+                w[L + "mlp.down"] = rnd(d, f, std=f ** -0.5)
+            else:
+                f = ml["expert"]["ff"]
+                for e in range(ml["router"]["experts"]):
+                    # pre-activations on both sides of the limit
+                    w[f"{L}mlp.e{e}.gate"], w[f"{L}mlp.e{e}.up"] = rnd(f, d, std=1.5 * d ** -0.5), rnd(f, d, std=1.5 * d ** -0.5)
+                    w[f"{L}mlp.e{e}.down"] = rnd(d, f, std=f ** -0.5)
+                w[L + "mlp.router"] = rnd(ml["router"]["experts"], d, std=2 * d ** -0.5)
+        if sd:
+            w[L + "side.gate"], w[L + "side.proj"] = rnd(sd, d, std=d ** -0.5), rnd(d, sd, std=sd ** -0.5)
+            w[L + "side.norm"] = rnd(d, std=0.1, mean=0.5)
+    return w
