@@ -20,7 +20,8 @@ Modes (``--mode``):
 * ``arch`` - not the headline: prefill and decode tokens/s of a layer-list design beside its closest
   existing model at equal layer sizes (engine/arch_bench.py; ``--arch-design dunesun``: beside a
   Mixtral-style model, ``kisutar``: beside an all-attention Dunesun model, ``bitonex``: beside a Dunesun
-  model of attention and Mamba-2 layers), one GPU, random weights.
+  model of attention and Mamba-2 layers, ``levovik``: beside a Dunesun model with an attention and a Mamba-2
+  layer for each of its layers), one GPU, random weights.
 ``--production``: the server runs with the reference's timeouts (15 s write, 30 s llm.timeout)
 instead of the bench's 600 s; answers that reach the deadline come back truncated
 (finish_reason "deadline") and overload as 503 - both are counted in the JSON line.
@@ -71,7 +72,7 @@ def parse(argv=None):
     ap.add_argument("--arch-seqs", type=int, default=4, help="arch: prompts in the prefill step")
     ap.add_argument("--arch-window", type=int, default=1024, help="arch: the Dunesun attention layers' window")
     ap.add_argument("--arch-which", choices=["both", "new", "ref"], default="both")
-    ap.add_argument("--arch-design", choices=["dunesun", "kisutar", "bitonex"], default="dunesun",
+    ap.add_argument("--arch-design", choices=["dunesun", "kisutar", "bitonex", "levovik"], default="dunesun",
                     help="arch: the layer-list design to measure beside its closest existing model")
     ap.add_argument("--rate", type=float, default=16.0, help="poisson: arrivals per second per replica")
     ap.add_argument("--production", action="store_true",

@@ -5,7 +5,10 @@ an all-attention Dunesun model (windowed attention with sinks, fp32 residual str
 with a shared expert in every layer - the same kernels family); Bitonex (rotary attention, linear
 attention and latent attention layers in turn, dense gated feed-forward) beside a Dunesun model of
 attention and Mamba-2 layers with the same heads, head sizes, recurrent state size and feed-forward
-width (one expert, so every token takes it).  Both models run through the same
+width (one expert, so every token takes it); Levovik (softmax attention beside gated linear attention
+or the gated delta rule in every layer, routed clamped experts) beside a Dunesun model that has one
+attention layer with the same experts and one Mamba-2 layer of equal state size for every Levovik
+layer.  Both models run through the same
 ModelRunner step functions the engine uses: one prefill step of ``seqs`` whole prompts, then decode
 steps of ``batch`` sequences (hipGraph replay where the model's decode is captured)."""
 from __future__ import annotations
@@ -120,7 +123,53 @@ def _bitonex_pair(size: str, window: int) -> tuple:
     return new, ref
 
 
-PAIRS = {"dunesun": _pair, "kisutar": _kisutar_pair, "bitonex": _bitonex_pair}
+# Levovik: (name, width, heads, kv heads, head dim, rotating dims, recurrent heads, key dim, value dim, low rank,
+#           experts, top, expert ff, dense ff, token-input dim, layers)
+LEVOVIK_SIZES = {
+    "s": ("d1024", 1024, 8, 2, 128, 64, 8, 128, 128, 64, 8, 2, 1024, 2816, 128, 4),
+    "m": ("d2048", 2048, 16, 4, 128, 64, 16, 128, 128, 64, 8, 2, 2048, 5632, 256, 4),
+    "l": ("d4096", 4096, 32, 8, 128, 64, 32, 128, 128, 128, 8, 2, 3584, 11008, 256, 2),
+}
+
+
+def _levovik_pair(size: str, window: int) -> tuple:
+    """Levovik (gated-linear and delta-rule layers in turn, the first feed-forward dense, the others
+    routed in two groups) and a Dunesun model with, for every Levovik layer, an attention layer over the
+    whole prefix with the same experts and a Mamba-2 layer with as many state entries per token."""
+    name, d, H, G, D, rd, Hr, dk, dv, rank, E, K, ff, fd, side, L = LEVOVIK_SIZES[size]
+    flat = lambda m: tuple(sorted(m.items()))
+    rot = {"rot.dims": rd, "rot.base": 5e5, "rot.scaling.factor": 8.0, "rot.scaling.low": 1.0, "rot.scaling.high": 4.0,
+           "rot.scaling.original": 8192}
+
+    def layer(i):
+        left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, **rot}
+        if i % 2 == 0:
+            kind, right = "parallel_2", {"heads": Hr, "dim": dk, "vdim": dv, "tau": 16.0, "a_rank": rank}
+        else:
+            kind, right = "parallel", {"heads": Hr, "kv_heads": max(1, Hr // 2), "dim": dk, "vdim": dv, "conv": 4, "a_rank": rank,
+                                       "g_rank": rank}
+        m = {"left_scale": 0.8, "right_scale": 1.1}
+        m.update({"left." + k: v for k, v in left.items()})
+        m.update({"right." + k: v for k, v in right.items()})
+        mlp = DenseSpec(fd) if i == 0 else MoESpec(E, K, ff, 0, limit=7.0, groups=2, keep_groups=1, route_scale=2.0)
+        return LayerSpec(kind, flat(m), mlp)
+
+    new = HybridConfig(name=f"levovik-{name}", arch="levovik", vocab_size=32000, d_model=d,
+                       layers=tuple(layer(i) for i in range(L)), max_position=8192, norm_eps=1e-5, logit_scale=0.5,
+                       embed_scale=float(d) ** 0.5, side_dim=side)
+    att = lambda mlp: LayerSpec("attention", flat({"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask.size": 0,
+                                                   "scale": D ** -0.5}), mlp)
+    ssm = LayerSpec("mamba2", flat({"heads": Hr * dv // 64, "vdim": 64, "state": dk, "groups": 1, "conv": 4,
+                                    "norm_groups": 1}), None)
+    ref_layers = []
+    for i in range(L):
+        ref_layers += [att(MoESpec(1, 1, fd, 0) if i == 0 else MoESpec(E, K, ff, 0)), ssm]
+    ref = HybridConfig(name=f"dunesun-pairs-{name}", arch="dunesun", vocab_size=32000, d_model=d, layers=tuple(ref_layers),
+                       max_position=8192)
+    return new, ref
+
+
+PAIRS = {"dunesun": _pair, "kisutar": _kisutar_pair, "bitonex": _bitonex_pair, "levovik": _levovik_pair}
 
 
 def _measure(cfg, seqs: int, prompt: int, batch: int, steps: int, warmup: int, graphs: bool) -> dict:

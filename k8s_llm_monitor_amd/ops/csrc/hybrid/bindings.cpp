@@ -21,7 +21,8 @@ int k8sllm_hy_rotary_norm_cache(void* qkv, long stride, long T, int Hq, int G, i
 int k8sllm_hy_decay_scan(float* o, const void* qkv, long stride, int q_col, int k_col, int v_col, const void* z,
                          long z_stride, const float* z_bias, const float* a_log, float inv_tau, const void* beta,
                          long b_stride, float* state, const int* cu, const int* ctx, const int* slot, int S, int H, int Gk,
-                         int dk, int dv, float q_scale, int unit, int f32, hipStream_t s);
+                         int dk, int dv, float q_scale, int unit, int f32, float* ws, long T, hipStream_t s);
+long k8sllm_hy_decay_scan_ws(long T, int H, int Gk, int dk);
 int k8sllm_hy_router_grouped(int* ids, float* wts, const void* h, long T, int d, const float* wr, int E, int K,
                              int groups, int keep, float scale, int f32, hipStream_t s);
 int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const void* a1, int t1, const void* a2,
@@ -607,9 +608,10 @@ void rotary_norm_cache(Tensor qkv, int64_t Hq, int64_t G, int64_t dk, int64_t dv
 }
 
 // The per-channel-decay recurrence (optionally with the delta rule: beta given); see decay_scan.hip
+// ws: fp32 workspace of decay_scan_ws(T, ...) floats - given, the two-launch form for prompts runs
 void decay_scan(Tensor o, Tensor qkv, int64_t q_col, int64_t k_col, int64_t v_col, Tensor z, Tensor z_bias, OptT a_log,
                 double tau, OptT beta, int64_t beta_col, Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t H,
-                int64_t Gk, int64_t dk, int64_t dv, double q_scale, bool unit) {
+                int64_t Gk, int64_t dk, int64_t dv, double q_scale, bool unit, OptT ws) {
   const int f = act(qkv, "qkv");
   same(z, f, "z");
   f32c(o, "o");
@@ -640,10 +642,16 @@ void decay_scan(Tensor o, Tensor qkv, int64_t q_col, int64_t k_col, int64_t v_co
     bp = (const char*)beta->data_ptr() + beta_col * beta->element_size();
     bstride = beta->stride(0);
   }
+  float* wp = nullptr;
+  if (ws.has_value()) {
+    f32c(*ws, "workspace");
+    TORCH_CHECK(ws->numel() >= k8sllm_hy_decay_scan_ws(T, (int)H, (int)Gk, (int)dk), "decay_scan: workspace too small");
+    wp = ws->data_ptr<float>();
+  }
   check(k8sllm_hy_decay_scan(o.data_ptr<float>(), qkv.data_ptr(), qkv.stride(0), (int)q_col, (int)k_col, (int)v_col,
                              z.data_ptr(), z.stride(0), z_bias.data_ptr<float>(), ap, (float)(1.0 / tau), bp, bstride,
                              state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
-                             (int)ctx.numel(), (int)H, (int)Gk, (int)dk, (int)dv, (float)q_scale, unit, f, cur()),
+                             (int)ctx.numel(), (int)H, (int)Gk, (int)dk, (int)dv, (float)q_scale, unit, f, wp, (long)T, cur()),
         "decay_scan");
 }
 

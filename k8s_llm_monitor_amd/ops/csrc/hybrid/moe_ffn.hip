@@ -117,24 +117,63 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
   }
 }
 
-// Sigmoid router with a choice restricted to the best groups.  One workgroup per token: wave w computes the
-// logits of experts w, w + 4, ... (fp32 weights, h widened), thread 0 scores the groups and picks.
-template <typename T>
+// Sigmoid router with a choice restricted to the best groups.  One workgroup per token computes the logits
+// (fp32 weights, h widened; NACC as in hy_router_kernel), thread 0 scores the groups and picks.
+template <typename T, int NACC>
 __global__ __launch_bounds__(256) void hy_router_grouped_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                                 const T* __restrict__ h, int d,
                                                                 const float* __restrict__ wr, int E, int K, int groups,
                                                                 int keep, float scale) {
   __shared__ float sc[kMaxE];
   __shared__ float gsc[kMaxE];
+  __shared__ float part[4][NACC > 0 ? NACC : 1];
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* x = h + t * d;
-  for (int e = wave; e < E; e += 4) {
-    const float* w = wr + (long)e * d;
-    float a = 0.f;
-    for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
-    a = wave_sum(a);
-    if (lane == 0) sc[e] = 1.f / (1.f + expf(-a));
+  if (NACC > 0) {  // at most NACC experts: h is read once, every expert's partial sum stays in a register
+    float acc[NACC > 0 ? NACC : 1];
+#pragma unroll
+    for (int e = 0; e < NACC; ++e) acc[e] = 0.f;
+    if ((d & 7) == 0) {
+      for (int c = threadIdx.x * 8; c < d; c += 2048) {
+        float xv[8];
+        load8(x + c, xv);
+#pragma unroll
+        for (int e = 0; e < NACC; ++e)
+          if (e < E) {
+            const float4 wa = *reinterpret_cast<const float4*>(wr + (long)e * d + c);
+            const float4 wb = *reinterpret_cast<const float4*>(wr + (long)e * d + c + 4);
+            acc[e] += xv[0] * wa.x + xv[1] * wa.y + xv[2] * wa.z + xv[3] * wa.w + xv[4] * wb.x + xv[5] * wb.y +
+                      xv[6] * wb.z + xv[7] * wb.w;
+          }
+      }
+    } else {
+#pragma unroll 4
+      for (int c = threadIdx.x; c < d; c += 256) {
+        const float xv = ldf(x + c);
+#pragma unroll
+        for (int e = 0; e < NACC; ++e)
+          if (e < E) acc[e] += xv * wr[(long)e * d + c];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < NACC; ++e) {
+      const float v = wave_sum(acc[e]);
+      if (lane == 0) part[wave][e] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < E) {
+      const int e = threadIdx.x;
+      sc[e] = 1.f / (1.f + expf(-(part[0][e] + part[1][e] + part[2][e] + part[3][e])));
+    }
+  } else {
+    for (int e = wave; e < E; e += 4) {
+      const float* w = wr + (long)e * d;
+      float a = 0.f;
+      for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
+      a = wave_sum(a);
+      if (lane == 0) sc[e] = 1.f / (1.f + expf(-a));
+    }
   }
   __syncthreads();
   const int per = E / groups;
@@ -405,12 +444,15 @@ int k8sllm_hy_router_grouped(int* ids, float* wts, const void* h, long T, int d,
   if (E > kMaxE || K > kMaxK || K < 1 || groups < 1 || E % groups || keep < 1 || keep > groups ||
       K > keep * (E / groups))
     return -1;
-  if (f32)
-    hipLaunchKernelGGL(hy_router_grouped_kernel<float>, dim3(T), dim3(256), 0, s, ids, wts, (const float*)h, d, wr, E, K,
-                       groups, keep, scale);
-  else
-    hipLaunchKernelGGL(hy_router_grouped_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, wts, (const bf16_t*)h, d, wr, E, K,
-                       groups, keep, scale);
+#define K8SLLM_RG(T_, NACC)                                                                                        \
+  hipLaunchKernelGGL((hy_router_grouped_kernel<T_, NACC>), dim3(T), dim3(256), 0, s, ids, wts, (const T_*)h, d, wr, E, K, \
+                     groups, keep, scale)
+  if (f32) {
+    if (E <= 8) K8SLLM_RG(float, 8); else if (E <= 16) K8SLLM_RG(float, 16); else K8SLLM_RG(float, 0);
+  } else {
+    if (E <= 8) K8SLLM_RG(bf16_t, 8); else if (E <= 16) K8SLLM_RG(bf16_t, 16); else K8SLLM_RG(bf16_t, 0);
+  }
+#undef K8SLLM_RG
   return (int)hipGetLastError();
 }
 

@@ -133,6 +133,40 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(T* __restrict__ o
   }
 }
 
+// The norm-first forms (after 1 / 2) with small groups (a head's values): one wave per (row, group), the
+// group's at most 64 NPL values in registers, so y is read once and no workgroup barrier is needed.
+template <typename T, int NPL>
+__global__ __launch_bounds__(256) void group_norm_gate_wave_kernel(T* __restrict__ out, const float* __restrict__ y,
+                                                                   const T* __restrict__ z, long z_stride,
+                                                                   const float* __restrict__ w, long rows, int n,
+                                                                   int groups, float eps, int after) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long idx = (long)blockIdx.x * 4 + wave;
+  if (idx >= rows * groups) return;
+  const long row = idx / groups;
+  const int g = (int)(idx - row * groups), gs = n / groups;
+  const float* yr = y + row * n + (long)g * gs;
+  const T* zr = z + row * z_stride + (long)g * gs;
+  float v[NPL], gt[NPL];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    const int c = lane + 64 * i;
+    v[i] = c < gs ? yr[c] : 0.f;
+    gt[i] = c < gs ? ldf(zr + c) : 0.f;
+    ss += v[i] * v[i];
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    const int c = lane + 64 * i;
+    if (c < gs)
+      stf(out + row * n + (long)g * gs + c,
+          v[i] * inv * w[(long)g * gs + c] * (after == 2 ? silu_f(gt[i]) : sigmoid_f(gt[i])));
+  }
+}
+
 // residual += mult * y * sigmoid(gate + bias), then the RMSNorm of the new residual times w.  y: any
 // float dtype, contiguous; gate: activation dtype, rows g_stride apart (a column range of a wider
 // projection).  Sum, sigmoid and norm are fp32.
@@ -567,6 +601,20 @@ int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_
                                int n, int groups, float eps, int after, int f32, hipStream_t s) {
   if (rows <= 0) return 0;
   if (groups < 1 || n % groups) return -1;
+  const int gs = n / groups;
+  if (after && groups > 1 && gs <= 256) {  // per-head norms: a wave per group
+    const dim3 grid((unsigned)((rows * groups + 3) / 4));
+#define K8SLLM_GW(T_, NPL)                                                                                         \
+  hipLaunchKernelGGL((group_norm_gate_wave_kernel<T_, NPL>), grid, dim3(256), 0, s, (T_*)out, y, (const T_*)z, z_stride, \
+                     w, rows, n, groups, eps, after)
+    if (f32) {
+      if (gs <= 64) K8SLLM_GW(float, 1); else if (gs <= 128) K8SLLM_GW(float, 2); else K8SLLM_GW(float, 4);
+    } else {
+      if (gs <= 64) K8SLLM_GW(bf16_t, 1); else if (gs <= 128) K8SLLM_GW(bf16_t, 2); else K8SLLM_GW(bf16_t, 4);
+    }
+#undef K8SLLM_GW
+    return (int)hipGetLastError();
+  }
   if (f32)
     hipLaunchKernelGGL(gated_group_norm_kernel<float>, dim3(rows, groups), dim3(256), 0, s, (float*)out, y,
                        (const float*)z, z_stride, w, n, groups, eps, after);

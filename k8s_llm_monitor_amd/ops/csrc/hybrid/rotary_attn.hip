@@ -13,7 +13,8 @@
 //                  (fp32, eps inside the root): norm == 1 before the turn, times qw / kw [dk]; norm == 2 after
 //                  the turn, no weight; norm == 0 none.  v_from_k: the row has no value columns and the value
 //                  pages take the keys as projected (before norm and turn; dv == dk).  One wave per head, the
-//                  head staged in LDS as fp32; the result is rounded to the activation dtype once.
+//                  head staged in LDS as fp32; the token's sines and cosines are evaluated once for all its
+//                  heads; the result is rounded to the activation dtype once.
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -29,7 +30,7 @@ __global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ 
                                                                 const float* __restrict__ q_scale,
                                                                 T* __restrict__ k_cache, T* __restrict__ v_cache,
                                                                 const int* __restrict__ slots, int bs, int v_from_k) {
-  extern __shared__ float heads[];  // [4 waves][dk]
+  extern __shared__ float heads[];  // [4 waves][dk], then the token's nf cosines and nf sines
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   T* row = qkv + t * stride;
@@ -37,6 +38,10 @@ __global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ 
   const float pos = (float)positions[t];
   const long slot = (slots != nullptr && k_cache != nullptr) ? slots[t] : -1;
   float* x = heads + wave * dk;
+  float* cst = heads + 4 * dk;
+  float* snt = cst + nf;
+  for (int i = threadIdx.x; i < nf; i += 256) sincosf(pos * freq[i], snt + i, cst + i);  // once for all heads
+  // (the first barrier below orders these writes before every read)
   for (int h0 = 0; h0 < Hq + G; h0 += 4) {  // query heads, then key heads: contiguous in the row
     // every wave makes every trip (the barriers below are the workgroup's); a wave without a head idles
     const int h = h0 + wave;
@@ -59,8 +64,7 @@ __global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ 
     __syncthreads();  // a lane turns pairs whose entries other lanes staged
     for (int i = lane; live && i < nf; i += 64) {
       const int a = pairs ? 2 * i : i, b = pairs ? 2 * i + 1 : i + nf;
-      float sn, cs;
-      sincosf(pos * freq[i], &sn, &cs);
+      const float sn = snt[i], cs = cst[i];
       const float u = x[a], v = x[b];
       x[a] = u * cs - v * sn;
       x[b] = v * cs + u * sn;
@@ -166,7 +170,7 @@ int k8sllm_hy_rotary_norm_cache(void* qkv, long stride, long T, int Hq, int G, i
   if (nf < 0 || 2 * nf > dk || Hq < 1 || G < 1 || dk > kMaxHeadDim || norm < 0 || norm > 2) return -1;
   if (norm == 1 && (qw == nullptr || kw == nullptr)) return -1;
   if (v_from_k && dv != dk) return -1;
-  const size_t lds = 4 * (size_t)dk * sizeof(float);
+  const size_t lds = (4 * (size_t)dk + 2 * (size_t)nf) * sizeof(float);
   if (f32)
     hipLaunchKernelGGL(rotary_norm_cache_kernel<float>, dim3(T), dim3(256), lds, s, (float*)qkv, stride, Hq, G, dk, dv,
                        positions, freq, nf, pairs, norm, qw, kw, eps, q_scale, (float*)k_cache, (float*)v_cache, slots, bs,

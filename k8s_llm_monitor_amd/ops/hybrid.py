@@ -711,7 +711,7 @@ def linear_attention(vkq: torch.Tensor, decay: torch.Tensor, state: torch.Tensor
 def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, z_bias: torch.Tensor,
                state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor, seg_slot: torch.Tensor, H: int, Gk: int,
                dk: int, dv: int, q_scale: float, a_log: Optional[torch.Tensor] = None, tau: float = 1.0,
-               beta: Optional[torch.Tensor] = None, beta_col: int = 0, unit: bool = False) -> torch.Tensor:
+               beta: Optional[torch.Tensor] = None, beta_col: int = 0, unit: bool = False, mode: int = 0) -> torch.Tensor:
     """Linear attention with a decay per head and key channel, optionally with the delta rule, as an
     fp32 recurrence over each segment.  Per head h (reading query / key head ``h // (H / Gk)``) and token:
 
@@ -728,7 +728,12 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
     ``beta_col + h`` holds head h's logit, ``beta_t = sigmoid(logit)``.  ``state`` [slots, H, dv, dk] fp32
     (a value row's key channels contiguous) is read at a segment's start (zero where seg_ctx is 0) and
     written back at its end.  Returns o [T, H*dv] fp32.  Decays, unit norms, gates, state, products and
-    sums are fp32."""
+    sums are fp32.
+
+    GPU: steps of prompts (a mean segment length of 32 rows or more) run as two launches - everything
+    that does not depend on the state (decays, unit norms, k . q, beta) for all rows at once into an fp32
+    workspace, then the recurrence over it; decode steps run as one launch.  ``mode`` 1 / 2 force the
+    one-launch / two-launch form (tests)."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         o = torch.zeros(T, H * dv, dtype=torch.float32)
@@ -765,8 +770,11 @@ def decay_scan(qkv: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.T
             state[slot] = S
         return o
     o = torch.empty(T, H * dv, dtype=torch.float32, device=qkv.device)
+    ws = None
+    if mode == 2 or (mode == 0 and T >= 32 * seg_slot.numel()):
+        ws = torch.empty(T * (2 * Gk * dk + H * dk + Gk + H), dtype=torch.float32, device=qkv.device)
     native().decay_scan(o, qkv, int(q_col), int(k_col), int(v_col), z, z_bias, a_log, float(tau), beta, int(beta_col),
-                        state, seg_cu, seg_ctx, seg_slot, int(H), int(Gk), int(dk), int(dv), float(q_scale), bool(unit))
+                        state, seg_cu, seg_ctx, seg_slot, int(H), int(Gk), int(dk), int(dv), float(q_scale), bool(unit), ws)
     return o
 
 

@@ -742,18 +742,29 @@ def test_gpu_new_ops_match_their_torch_forms(dtype):
         gate = (torch.randn(T, n, generator=g) * 2).to(dtype)
         c, u, _, _ = both(hops.gated_lookup, gate, table, ids, 5)
         close(u.cpu().float(), c.double(), tol=tol)
+    # a norm per head, then the gate: groups of a wave's width and less, more, and beyond the wave kernel
+    for T, groups, gs in ((5, 4, 32), (3, 3, 7), (4, 2, 128), (2, 2, 200), (3, 2, 300), (2, 16, 64), (2, 1, 48)):
+        n = groups * gs
+        yy, zz = torch.randn(T, n, generator=g) * 3, (torch.randn(T, n + 9, generator=g) * 2).to(dtype)
+        ww = torch.rand(n, generator=g) + 0.5
+        for gate in ("sigmoid", "silu"):
+            c, u, _, _ = both(hops.gated_group_norm, yy, zz, 9, ww, 1e-5, groups, dtype, True, gate)
+            close(u.cpu().float(), c.double(), tol=tol)
     z = (torch.randn(6, 40, generator=g) * 2).to(dtype)
     for col, f in ((8, 16), (3, 7)):
         for kind, lim in (("relu", 0.0), ("clamped_swish", 1.1)):
             c, u, _, _ = both(hops.glu, z, col, f, kind, lim)
             close(u.cpu().float(), c.double(), tol=tol)
     if dtype == torch.float32:
-        hh, wr = torch.randn(70, 24, generator=g), torch.randn(12, 24, generator=g)
-        for top, groups in ((3, (2, 1)), (2, (4, 2)), (4, (12, 5)), (5, (1, 1)), (1, (3, 3)), (12, (1, 1))):
-            (ic, wc), (ig, wg), _, _ = both(hops.moe_router_grouped, hh, wr, 12, top, *groups, 2.5)
-            oc, og = ic.long().argsort(-1), ig.cpu().long().argsort(-1)
-            assert torch.equal(ic.long().gather(1, oc), ig.cpu().long().gather(1, og))
-            close(wg.cpu().gather(1, og), wc.gather(1, oc).double(), tol=1e-5)
+        for E, d, cases in ((12, 24, ((3, (2, 1)), (2, (4, 2)), (4, (12, 5)), (5, (1, 1)), (1, (3, 3)), (12, (1, 1)))),
+                            (8, 21, ((2, (2, 1)), (8, (1, 1)))), (6, 40, ((3, (3, 2)),)), (24, 16, ((4, (4, 2)), (6, (8, 3)))),
+                            (16, 2056, ((4, (4, 2)),))):
+            hh, wr = torch.randn(70, d, generator=g), torch.randn(E, d, generator=g) * d ** -0.5
+            for top, groups in cases:
+                (ic, wc), (ig, wg), _, _ = both(hops.moe_router_grouped, hh, wr, E, top, *groups, 2.5)
+                oc, og = ic.long().argsort(-1), ig.cpu().long().argsort(-1)
+                assert torch.equal(ic.long().gather(1, oc), ig.cpu().long().gather(1, og))
+                close(wg.cpu().gather(1, og), wc.gather(1, oc).double(), tol=1e-5)
     # norm + rotation + page writes, both orders and layouts, rotating part smaller than the head
     for Hq, G, dk, dv, rd in ((4, 2, 12, 6, 8), (6, 1, 64, 64, 64), (6, 2, 128, 128, 32), (3, 3, 7, 5, 4)):
         T = 9
@@ -772,7 +783,7 @@ def test_gpu_new_ops_match_their_torch_forms(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,Gk,dk,dv", [(2, 2, 32, 32), (4, 2, 48, 32), (3, 1, 64, 96), (2, 2, 128, 128), (1, 1, 200, 40), (6, 3, 5, 7),
-                                        (2, 1, 16, 8), (1, 1, 1, 1), (2, 2, 256, 16)])
+                                        (2, 1, 16, 8), (1, 1, 1, 1), (2, 2, 256, 16), (2, 1, 12, 70), (3, 3, 36, 130), (2, 2, 100, 9)])
 @pytest.mark.parametrize("delta_rule", [True, False], ids=["delta", "plain"])
 def test_gpu_decay_scan_matches_the_recurrence(H, Gk, dk, dv, delta_rule):
     """The scan kernel against the float64 recurrence and the torch form: segments shorter than, equal
@@ -792,14 +803,16 @@ def test_gpu_decay_scan_matches_the_recurrence(H, Gk, dk, dv, delta_rule):
     args = (0, Gk * dk, 2 * Gk * dk)
     want_state = st.clone()
     want = hops.decay_scan(qkv, *args, z, zb, want_state, cu, ctx, slot, H, Gk, dk, dv, dk ** -0.5, **kw)
-    got_state = st.to("cuda")
     gk = {k: (v.to("cuda") if isinstance(v, torch.Tensor) else v) for k, v in kw.items()}
-    got = hops.decay_scan(qkv.to("cuda"), *args, z.to("cuda"), zb.to("cuda"), got_state, cu.to("cuda"), ctx.to("cuda"),
-                          slot.to("cuda"), H, Gk, dk, dv, dk ** -0.5, **gk)
-    close(got.cpu(), want.double(), tol=2e-5)
-    close(got_state.cpu(), want_state.double(), tol=2e-5)
     a, b = int(cu[4]), int(cu[5])  # the 100-token segment starts from zero: the written-out recurrence
-    close(got[a:b].cpu(), _scan_want(qkv[a:b], z[a:b], zb, a_log, H, Gk, dk, dv, delta_rule, 3.0), tol=2e-5)
+    alone = _scan_want(qkv[a:b], z[a:b], zb, a_log, H, Gk, dk, dv, delta_rule, 3.0)
+    for mode in (1, 2):  # the one-launch form and the two-launch form for prompts
+        got_state = st.to("cuda")
+        got = hops.decay_scan(qkv.to("cuda"), *args, z.to("cuda"), zb.to("cuda"), got_state, cu.to("cuda"), ctx.to("cuda"),
+                              slot.to("cuda"), H, Gk, dk, dv, dk ** -0.5, mode=mode, **gk)
+        close(got.cpu(), want.double(), tol=2e-5)
+        close(got_state.cpu(), want_state.double(), tol=2e-5)
+        close(got[a:b].cpu(), alone, tol=2e-5)
 
 
 @pytest.mark.gpu
