@@ -74,11 +74,12 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(float* __restrict__ o, 
   if (t1 <= t0) return;
   const int n0 = chunk * 8;
   const int g = h / (H / Gk);
-  for (int i = threadIdx.x; i < TB * ROW; i += 256) {  // channels beyond dk stay zero
-    (&qs[0][0])[i] = 0.f;
-    (&ks[0][0])[i] = 0.f;
-    (&gs[0][0])[i] = 0.f;
-  }
+  if (dk != 8 * CH)  // channels beyond dk stay zero (none where the lanes' 8-channel chunks cover dk exactly)
+    for (int i = threadIdx.x; i < min(TB, t1 - t0) * ROW; i += 256) {
+      (&qs[0][0])[i] = 0.f;
+      (&ks[0][0])[i] = 0.f;
+      (&gs[0][0])[i] = 0.f;
+    }
   float S[8];
   float* sp = state + (((long)sl * H + h) * dv + p) * dk + n0;
   const bool carried = ctx[s] > 0;
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(float* __restrict__ o, 
 // ---- the two-launch form for prompts
 // workspace rows (fp32): qn, kn [T][Gk][dk], gd [T][H][dk], kq [T][Gk], bt [T][H]
 template <typename T>
-__global__ __launch_bounds__(128) void decay_prep_kernel(float* __restrict__ qn, float* __restrict__ kn,
+__global__ __launch_bounds__(256) void decay_prep_kernel(float* __restrict__ qn, float* __restrict__ kn,
                                                          float* __restrict__ gd, float* __restrict__ kq,
                                                          float* __restrict__ bt, const T* __restrict__ qkv, long stride,
                                                          int q_col, int k_col, const T* __restrict__ z, long z_stride,
@@ -191,41 +192,44 @@ __global__ __launch_bounds__(128) void decay_prep_kernel(float* __restrict__ qn,
                                                          const float* __restrict__ a_log, float inv_tau,
                                                          const T* __restrict__ beta, long b_stride, int H, int Gk,
                                                          int dk, float q_scale, int unit) {
-  __shared__ float red[2];
+  // one workgroup per token: the decays of all heads, beta, then a wave per query / key head
   const long t = blockIdx.x;
-  const int y = blockIdx.y;
-  if (y < H) {  // head y: its decays and its beta
-    const float A = a_log != nullptr ? expf(a_log[y]) : 0.f;
-    for (int n = threadIdx.x; n < dk; n += 128) {
-      const float zz = ldf(z + t * z_stride + (long)y * dk + n) + z_bias[y * dk + n];
-      gd[(t * H + y) * dk + n] = a_log != nullptr ? expf(-A * softplus_f(zz)) : expf(-softplus_f(-zz) * inv_tau);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nd = H * dk;
+  const T* zr = z + t * z_stride;
+  float* gr = gd + t * nd;
+  if (a_log != nullptr) {
+    for (int e = threadIdx.x; e < nd; e += 256)
+      gr[e] = expf(-expf(a_log[e / dk]) * softplus_f(ldf(zr + e) + z_bias[e]));
+  } else {
+    for (int e = threadIdx.x; e < nd; e += 256) gr[e] = expf(-softplus_f(-(ldf(zr + e) + z_bias[e])) * inv_tau);
+  }
+  if (beta != nullptr)
+    for (int h = threadIdx.x; h < H; h += 256) bt[t * H + h] = sigmoid_f(ldf(beta + t * b_stride + h));
+  for (int g = wave; g < Gk; g += 4) {
+    const T* row = qkv + t * stride + (long)g * dk;
+    float sq = 0.f, sk = 0.f;
+    if (unit) {
+      for (int n = lane; n < dk; n += 64) {
+        const float q = ldf(row + q_col + n), k = ldf(row + k_col + n);
+        sq += q * q;
+        sk += k * k;
+      }
+      sq = wave_sum(sq);
+      sk = wave_sum(sk);
     }
-    if (beta != nullptr && threadIdx.x == 0) bt[t * H + y] = sigmoid_f(ldf(beta + t * b_stride + y));
-    return;
-  }
-  const int g = y - H;  // query / key head g
-  const T* row = qkv + t * stride + (long)g * dk;
-  float sq = 0.f, sk = 0.f;
-  if (unit) {
-    for (int n = threadIdx.x; n < dk; n += 128) {
-      const float q = ldf(row + q_col + n), k = ldf(row + k_col + n);
-      sq += q * q;
-      sk += k * k;
+    const float mq = unit ? q_scale / sqrtf(sq + 1e-6f) : q_scale;
+    const float mk = unit ? 1.0f / sqrtf(sk + 1e-6f) : 1.f;
+    float dot = 0.f;
+    for (int n = lane; n < dk; n += 64) {
+      const float q = ldf(row + q_col + n) * mq, k = ldf(row + k_col + n) * mk;
+      qn[(t * Gk + g) * dk + n] = q;
+      kn[(t * Gk + g) * dk + n] = k;
+      dot += q * k;
     }
-    sq = block_sum<128>(sq, red);
-    sk = block_sum<128>(sk, red);
+    dot = wave_sum(dot);
+    if (lane == 0) kq[t * Gk + g] = dot;
   }
-  const float mq = unit ? q_scale / sqrtf(sq + 1e-6f) : q_scale;
-  const float mk = unit ? 1.0f / sqrtf(sk + 1e-6f) : 1.f;
-  float dot = 0.f;
-  for (int n = threadIdx.x; n < dk; n += 128) {
-    const float q = ldf(row + q_col + n) * mq, k = ldf(row + k_col + n) * mk;
-    qn[(t * Gk + g) * dk + n] = q;
-    kn[(t * Gk + g) * dk + n] = k;
-    dot += q * k;
-  }
-  dot = block_sum<128>(dot, red);
-  if (threadIdx.x == 0) kq[t * Gk + g] = dot;
 }
 
 template <typename T, int CH, bool DELTA>
@@ -412,7 +416,7 @@ static int launch_decay_staged(float* o, const void* qkv, long stride, int q_col
   float* gd = kn + rows * Gk * dk;
   float* kq = gd + rows * H * dk;
   float* bt = kq + rows * Gk;
-  hipLaunchKernelGGL(decay_prep_kernel<T>, dim3((unsigned)rows, (unsigned)(H + Gk)), dim3(128), 0, s, qn, kn, gd, kq, bt,
+  hipLaunchKernelGGL(decay_prep_kernel<T>, dim3((unsigned)rows), dim3(256), 0, s, qn, kn, gd, kq, bt,
                      (const T*)qkv, stride, q_col, k_col, (const T*)z, z_stride, z_bias, a_log, inv_tau, (const T*)beta,
                      b_stride, H, Gk, dk, q_scale, unit);
 #define K8SLLM_DS(CH)                                                                                                  \

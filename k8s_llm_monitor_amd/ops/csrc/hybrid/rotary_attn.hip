@@ -41,16 +41,16 @@ __global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ 
   float* cst = heads + 4 * dk;
   float* snt = cst + nf;
   for (int i = threadIdx.x; i < nf; i += 256) sincosf(pos * freq[i], snt + i, cst + i);  // once for all heads
-  // (the first barrier below orders these writes before every read)
-  for (int h0 = 0; h0 < Hq + G; h0 += 4) {  // query heads, then key heads: contiguous in the row
-    // every wave makes every trip (the barriers below are the workgroup's); a wave without a head idles
-    const int h = h0 + wave;
-    const bool live = h < Hq + G;
+  __syncthreads();
+  // query heads, then key heads (contiguous in the row), a wave per head.  x is this wave's own LDS row: a
+  // wave's LDS instructions execute in issue order, so a wave barrier (no reordering by the compiler) is all
+  // that lanes reading what other lanes of the wave wrote need.
+  for (int h = wave; h < Hq + G; h += 4) {
     T* hd = row + (long)h * dk;
     const bool is_k = h >= Hq;
     const int g = h - Hq;
     float ss = 0.f;
-    for (int c = lane; live && c < dk; c += 64) {
+    for (int c = lane; c < dk; c += 64) {
       const float v = ldf(hd + c);
       x[c] = v;
       ss += v * v;
@@ -59,31 +59,32 @@ __global__ __launch_bounds__(256) void rotary_norm_cache_kernel(T* __restrict__ 
     if (norm == 1) {
       const float inv = 1.0f / sqrtf(wave_sum_dpp(ss) / (float)dk + eps);
       const float* w = is_k ? kw : qw;
-      for (int c = lane; live && c < dk; c += 64) x[c] = x[c] * inv * w[c];
+      for (int c = lane; c < dk; c += 64) x[c] = x[c] * inv * w[c];
     }
-    __syncthreads();  // a lane turns pairs whose entries other lanes staged
-    for (int i = lane; live && i < nf; i += 64) {
+    __builtin_amdgcn_wave_barrier();  // a lane turns pairs whose entries other lanes staged
+    for (int i = lane; i < nf; i += 64) {
       const int a = pairs ? 2 * i : i, b = pairs ? 2 * i + 1 : i + nf;
       const float sn = snt[i], cs = cst[i];
       const float u = x[a], v = x[b];
       x[a] = u * cs - v * sn;
       x[b] = v * cs + u * sn;
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     float mul = 1.f;
     if (norm == 2) {
       float s2 = 0.f;
-      for (int c = lane; live && c < dk; c += 64) s2 += x[c] * x[c];
+      for (int c = lane; c < dk; c += 64) s2 += x[c] * x[c];
       mul = 1.0f / sqrtf(wave_sum_dpp(s2) / (float)dk + eps);
     }
-    if (live && !is_k && q_scale != nullptr) mul *= q_scale[h];
-    T* kp = (live && is_k && slot >= 0) ? k_cache + slot * (long)nk + (long)g * dk : nullptr;
-    for (int c = lane; live && c < dk; c += 64) {
+    if (!is_k && q_scale != nullptr) mul *= q_scale[h];
+    T* kp = (is_k && slot >= 0) ? k_cache + slot * (long)nk + (long)g * dk : nullptr;
+    for (int c = lane; c < dk; c += 64) {
       stf(hd + c, x[c] * mul);
       if (kp != nullptr) kp[c] = hd[c];
     }
-    __syncthreads();  // the next head reuses x
+    __builtin_amdgcn_wave_barrier();  // the next head reuses x
   }
+  __syncthreads();  // the value copy below reads nothing the loop wrote, but keeps the workgroup together
   if (!v_from_k && slot >= 0)
     for (int c = threadIdx.x; c < nv; c += 256) v_cache[((slot / bs) * nv + c) * bs + slot % bs] = row[nq + nk + c];
 }
