@@ -134,7 +134,7 @@ LEVOVIK_SIZES = {
 
 def _levovik_pair(size: str, window: int) -> tuple:
     """Levovik (gated-linear and delta-rule layers in turn, the first feed-forward dense, the others
-    routed in two groups) and a Dunesun model with, for every Levovik layer, an attention layer over the
+    routed in four groups) and a Dunesun model with, for every Levovik layer, an attention layer over the
     whole prefix with the same experts and a Mamba-2 layer with as many state entries per token."""
     name, d, H, G, D, rd, Hr, dk, dv, rank, E, K, ff, fd, side, L = LEVOVIK_SIZES[size]
     flat = lambda m: tuple(sorted(m.items()))
@@ -144,18 +144,18 @@ def _levovik_pair(size: str, window: int) -> tuple:
     def layer(i):
         left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, **rot}
         if i % 2 == 0:
-            kind, right = "parallel_2", {"heads": Hr, "dim": dk, "vdim": dv, "tau": 16.0, "a_rank": rank}
+            kind, right = "parallel_2", {"heads": Hr, "dim": dk, "vdim": dv, "tau": 8.0, "a_rank": rank}
         else:
             kind, right = "parallel", {"heads": Hr, "kv_heads": max(1, Hr // 2), "dim": dk, "vdim": dv, "conv": 4, "a_rank": rank,
                                        "g_rank": rank}
-        m = {"left_scale": 0.8, "right_scale": 1.1}
+        m = {"left_scale": 1.0, "right_scale": 1.0}
         m.update({"left." + k: v for k, v in left.items()})
         m.update({"right." + k: v for k, v in right.items()})
-        mlp = DenseSpec(fd) if i == 0 else MoESpec(E, K, ff, 0, limit=7.0, groups=2, keep_groups=1, route_scale=2.0)
+        mlp = DenseSpec(fd) if i == 0 else MoESpec(E, K, ff, 0, limit=7.0, groups=4, keep_groups=2, route_scale=1.5)
         return LayerSpec(kind, flat(m), mlp)
 
     new = HybridConfig(name=f"levovik-{name}", arch="levovik", vocab_size=32000, d_model=d,
-                       layers=tuple(layer(i) for i in range(L)), max_position=8192, norm_eps=1e-5, logit_scale=0.5,
+                       layers=tuple(layer(i) for i in range(L)), max_position=8192, norm_eps=1e-5, logit_scale=0.7,
                        embed_scale=float(d) ** 0.5, side_dim=side)
     att = lambda mlp: LayerSpec("attention", flat({"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask.size": 0,
                                                    "scale": D ** -0.5}), mlp)

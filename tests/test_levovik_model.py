@@ -50,7 +50,7 @@ def gla(heads=3, dim=6, vdim=10, tau=4.0, a_rank=5):
     return {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "a_rank": a_rank}
 
 
-def par(left=None, right=None, ls=0.8, rs=1.1, mlp=None):
+def par(left=None, right=None, ls=0.9, rs=1.3, mlp=None):
     return {"type": "parallel", "mixer": {"left": left or att_a(), "right": right or delta(), "left_scale": ls,
                                           "right_scale": rs}, "mlp": mlp}
 
@@ -139,7 +139,7 @@ def test_layer_outputs_match_oracle():
 def test_ops_against_oracle_functions():
     g = torch.Generator().manual_seed(1)
     # frequencies: kept, blended and slowed entries, and no rescaling
-    for r in (rot(), rot(16, 5e5, 8.0, 512), rot(6, 10.0, 2.0, 8, 0.5, 3.0)):
+    for r in (rot(), rot(16, 3e5, 6.0, 384), rot(6, 10.0, 2.0, 8, 0.5, 3.0)):
         close(hops.rotary_freq(r["base"], r["dims"], scaling=r["scaling"]), O.scaled_frequencies(r), tol=1e-6)
     fr = O.scaled_frequencies(rot())
     plain = O.scaled_frequencies({"dims": 8, "base": 100.0})
@@ -148,8 +148,8 @@ def test_ops_against_oracle_functions():
     x, a, b, y = (torch.randn(5, 12, generator=g) for _ in range(4))
     w, wy = torch.rand(12, generator=g) + 0.5, torch.rand(12, generator=g)
     res = x.clone()
-    h = hops.sum_norm(res, ((a, 0.8), (b, 1.1)), (y, wy), w, 1e-5, True, False, torch.float32)
-    want = x.double() + 0.8 * a.double() + 1.1 * b.double() + O.rms(y.double(), 1e-5) * wy.double()
+    h = hops.sum_norm(res, ((a, 0.7), (b, 1.3)), (y, wy), w, 1e-5, True, False, torch.float32)
+    want = x.double() + 0.7 * a.double() + 1.3 * b.double() + O.rms(y.double(), 1e-5) * wy.double()
     close(res, want, tol=1e-6)
     close(h, O.layer_norm(want, w.double(), 1e-5), tol=1e-6)
     # the per-layer token input's gate
@@ -625,9 +625,9 @@ def test_gpu_odd_sizes(dtype):
         close(got, want) if dtype == torch.float32 else close_most(got, want, 0.06, frac=0.9)
 
 
-BIG = make_cfg([par2(att_b(8, 2, 64, 0.125, dims=64, base=5e5, original=64), gla(4, 64, 32, 16.0, 16), mlp=dense(192)),
+BIG = make_cfg([par2(att_b(8, 2, 64, 0.125, dims=64, base=5e5, original=64), gla(4, 64, 32, 12.0, 16), mlp=dense(192)),
                 par(att_a(4, 2, 128, 128, 0.09, dims=32, base=1e6, factor=8.0, original=64), delta(4, 2, 32, 64, 4, 16, 24),
-                    mlp=moe(8, 2, 64, 1.5, (2, 1), 2.0)),
+                    mlp=moe(8, 2, 64, 1.25, (4, 2), 1.75)),
                 par2(att_b(4, 4, 128, 0.09, dims=128, base=1e4, original=128), gla(2, 128, 64, 8.0, 8), mlp=moe(4, 2, 128, 1.0, None)),
                 par(att_a(8, 1, 64, 64, 0.125, dims=64, base=1e4, original=256), delta(2, 2, 128, 128, 4, 8, 8))],
                width=128, vocab=211, side=16)
@@ -726,7 +726,7 @@ def test_gpu_new_ops_match_their_torch_forms(dtype):
         x, a, b, y = torch.randn(T, n, generator=g), torch.randn(T, n, generator=g).to(dtype), torch.randn(T, n, generator=g), \
             torch.randn(T, n, generator=g).to(dtype)
         w, wy = torch.rand(n, generator=g) + 0.5, torch.rand(n, generator=g)
-        for center, wn, normed, adds in ((True, w, (y, wy), ((a, 0.8), (b, 1.1))), (False, w, None, ((a, 1.0),)),
+        for center, wn, normed, adds in ((True, w, (y, wy), ((a, 0.7), (b, 1.3))), (False, w, None, ((a, 1.0),)),
                                          (True, None, (y, wy), ()), (True, w, None, ())):
             def run(x_, *ts):
                 ts = list(ts)
