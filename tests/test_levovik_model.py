@@ -24,7 +24,7 @@ from k8s_llm_monitor_amd.models.config import get_config, hybrid_config_from_dic
 from k8s_llm_monitor_amd.models.hybrid import state_dict
 from k8s_llm_monitor_amd.models.registry import build_model, config_from_dir
 from k8s_llm_monitor_amd.ops import hybrid as hops
-from test_hybrid_model import ROOT, Rig, _save, close, close_most, toks
+from test_hybrid_model import ROOT, Rig, _save, close, toks
 
 
 # ------------------------------------------------------------------ small configurations
@@ -568,26 +568,49 @@ def test_trace_command_replays_steps(tmp_path):
 
 # ------------------------------------------------------------------ the same through the HIP kernels
 
-def _bf16_close(got, want):
-    close_most(got, want, 0.05, frac=0.9)
+def _row_err(got, want):
+    scale = float(want.pow(2).mean().sqrt())
+    return (got.double() - want).pow(2).mean(-1).sqrt() / scale
+
+
+def _bf16_ref_err(cfg, w, t, want, **kw):
+    """What bf16 rounding alone costs on this model and prompt: the torch forms on the CPU, in bf16,
+    against the oracle (row errors over the logits' scale)."""
+    return _row_err(rig_for(cfg, w=w, dtype=torch.bfloat16, **kw).run_cut("a", t, [len(t)]), want)
+
+
+def _bf16_close(got, want, ref_err):
+    """A bf16 run through the kernels is about as close to the oracle as the bf16 torch forms are: the
+    median and the 80th percentile of the row errors within 3 x theirs.  Both carry rounding noise of the
+    same size but not the same noise, and a sharply peaked softmax or a slowly decaying state downstream
+    amplifies one realisation two times more than another (measured on these configurations, in either
+    direction); a router decision that is a near tie falls either way in both.  A wrong state, page or
+    edge moves most rows by ten times the rounding level and more; the sharp comparisons are the fp32 ones."""
+    e = _row_err(got, want)
+    for q in (0.5, 0.8):
+        a, b = float(e.quantile(q)), float(ref_err.quantile(q))
+        assert a <= 3.0 * b + 2e-3, f"quantile {q}: {a:.3e} against {b:.3e} of the bf16 torch forms"
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gpu_cuts_and_batches_match_oracle(dtype):
-    cmp = close if dtype == torch.float32 else _bf16_close
     rig = rig_for(FULL, 6, device="cuda", dtype=dtype)
     t = toks(70, FULL["vocab"], 4)
-    want = O.forward(FULL, rig.w, t)
-    for cuts in ([70], [2, 2, 3, 16, 1, 31], [33, 2, 2, 2], []):
-        cmp(rig.run_cut("a", t, cuts), want)
     u = toks(40, FULL["vocab"], 8)
-    wu = O.forward(FULL, rig.w, u)
+    want, wu = O.forward(FULL, rig.w, t), O.forward(FULL, rig.w, u)
+    if dtype == torch.float32:
+        cmp = lambda got, ref, which: close(got, ref)
+    else:
+        errs = {"t": _bf16_ref_err(FULL, rig.w, t, want), "u": _bf16_ref_err(FULL, rig.w, u, wu)}
+        cmp = lambda got, ref, which: _bf16_close(got, ref, errs[which])
+    for cuts in ([70], [2, 2, 3, 16, 1, 31], [33, 2, 2, 2], []):
+        cmp(rig.run_cut("a", t, cuts), want, "t")
     a = rig.step([("a", t[:30]), ("b", u[:5])])
     b = rig.step([("a", t[30:31]), ("b", u[5:])], end=["b"])
     c = rig.step([("a", t[31:])], end=["a"])
-    cmp(torch.cat([a["a"], b["a"], c["a"]]), want)
-    cmp(torch.cat([a["b"], b["b"]]), wu)
+    cmp(torch.cat([a["a"], b["a"], c["a"]]), want, "t")
+    cmp(torch.cat([a["b"], b["b"]]), wu, "u")
 
 
 @pytest.mark.gpu
@@ -620,9 +643,10 @@ def test_gpu_odd_sizes(dtype):
     rig = rig_for(cfg, 31, device="cuda", dtype=dtype)
     t = toks(41, 53, 3)
     want = O.forward(cfg, rig.w, t)
+    ref = _bf16_ref_err(cfg, rig.w, t, want) if dtype == torch.bfloat16 else None
     for cuts in ([41], [3, 2, 17]):
         got = rig.run_cut("a", t, cuts)
-        close(got, want) if dtype == torch.float32 else close_most(got, want, 0.06, frac=0.9)
+        close(got, want) if dtype == torch.float32 else _bf16_close(got, want, ref)
 
 
 BIG = make_cfg([par2(att_b(8, 2, 64, 0.125, dims=64, base=5e5, original=64), gla(4, 64, 32, 12.0, 16), mlp=dense(192)),
@@ -640,8 +664,9 @@ def test_gpu_matrix_core_sizes_bf16():
     rig = rig_for(BIG, 6, device="cuda", dtype=torch.bfloat16, num_blocks=48)
     t = toks(150, BIG["vocab"], 4)
     want = O.forward(BIG, rig.w, t)
+    ref = _bf16_ref_err(BIG, rig.w, t, want, num_blocks=48)
     for cuts in ([150], [2, 2, 3, 16, 1, 31], [100]):
-        _bf16_close(rig.run_cut("a", t, cuts), want)
+        _bf16_close(rig.run_cut("a", t, cuts), want, ref)
     r32 = rig_for(BIG, 6, device="cuda", dtype=torch.float32, num_blocks=48)
     close(r32.run_cut("a", t, [70, 3]), want)
 
@@ -658,7 +683,7 @@ def test_gpu_long_prompt_fp32_and_bf16():
     close(r32.run_cut("a", t, [700]), want)
     close(r32.run_cut("a", t, [513, 180]), want)
     rig = rig_for(cfg, w=w, device="cuda", dtype=torch.bfloat16, num_blocks=96)
-    _bf16_close(rig.run_cut("a", t, [600, 95]), want)
+    _bf16_close(rig.run_cut("a", t, [600, 95]), want, _bf16_ref_err(cfg, w, t, want, num_blocks=96))
 
 
 @pytest.mark.gpu
