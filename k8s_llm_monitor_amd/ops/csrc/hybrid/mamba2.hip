@@ -90,16 +90,34 @@ __global__ __launch_bounds__(256) void conv_silu_vec8_kernel(T* __restrict__ out
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   }
-  for (int j = 0; j < taps; ++j) {
-    const int i = r - (taps - 1) + j;
-    if (i >= 0)
-      load8(proj + (long)(row - (taps - 1) + j) * stride + col0 + c, x);
-    else if (carried)
-      load8(state + ((long)sl * (taps - 1) + (taps - 1 + i)) * C + c, x);
-    else
-      continue;
+  if (taps == 4) {  // the usual width: a thread's 8 x 4 weights are 128 contiguous bytes, read as 16-byte loads
+    float4 wv[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) acc[k] += cw[(long)(c + k) * taps + j] * x[k];
+    for (int k = 0; k < 8; ++k) wv[k] = *reinterpret_cast<const float4*>(cw + (long)(c + k) * 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = r - 3 + j;
+      if (i >= 0)
+        load8(proj + (long)(row - 3 + j) * stride + col0 + c, x);
+      else if (carried)
+        load8(state + ((long)sl * 3 + (3 + i)) * C + c, x);
+      else
+        continue;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[k] += (j == 0 ? wv[k].x : j == 1 ? wv[k].y : j == 2 ? wv[k].z : wv[k].w) * x[k];
+    }
+  } else {
+    for (int j = 0; j < taps; ++j) {
+      const int i = r - (taps - 1) + j;
+      if (i >= 0)
+        load8(proj + (long)(row - (taps - 1) + j) * stride + col0 + c, x);
+      else if (carried)
+        load8(state + ((long)sl * (taps - 1) + (taps - 1 + i)) * C + c, x);
+      else
+        continue;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[k] += cw[(long)(c + k) * taps + j] * x[k];
+    }
   }
 #pragma unroll
   for (int k = 0; k < 8; ++k) acc[k] = silu_f(acc[k]);
