@@ -812,18 +812,18 @@ def test_gpu_new_ops_match_their_torch_forms(dtype):
 @pytest.mark.parametrize("delta_rule", [True, False], ids=["delta", "plain"])
 def test_gpu_decay_scan_matches_the_recurrence(H, Gk, dk, dv, delta_rule):
     """The scan kernel against the float64 recurrence and the torch form: segments shorter than, equal
-    to and longer than its 16-token tile, one continuing from its slot, one padding segment, a slot
+    to and longer than its 16- and 32-token tiles, some continuing from their slots, one padding segment, a slot
     with leftovers that a starting sequence must not see; outputs and the states left in the slots."""
     g = torch.Generator().manual_seed(5)
     if not delta_rule:
         Gk = H
-    lens = [1, 15, 16, 17, 100, 7, 40]
+    lens = [1, 15, 16, 17, 100, 7, 33, 32, 31]
     cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
-    ctx = torch.tensor([0, 5, 0, 64, 0, 3, 9], dtype=torch.int32)
-    slot = torch.tensor([0, 1, 2, 3, 4, -1, 5], dtype=torch.int32)
+    ctx = torch.tensor([0, 5, 0, 64, 0, 3, 9, 0, 2], dtype=torch.int32)
+    slot = torch.tensor([0, 1, 2, 3, 4, -1, 5, 7, 6], dtype=torch.int32)
     T = int(cu[-1])
     qkv, z, zb, a_log = _scan_inputs(g, T, H, Gk, dk, dv)
-    st = torch.randn(6, H, dv, dk, generator=g) * 0.3
+    st = torch.randn(8, H, dv, dk, generator=g) * 0.3
     kw = dict(a_log=a_log, beta=qkv, beta_col=2 * Gk * dk + H * dv, unit=True) if delta_rule else dict(tau=3.0)
     args = (0, Gk * dk, 2 * Gk * dk)
     want_state = st.clone()
